@@ -1,0 +1,321 @@
+/*
+ * tbv_oracle.c -- CPU restatement of the reference's on-GPU all-reduce data path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker: tests, the smoke check and
+ * the bench's cpu_baseline leg link it.  The shipped library never calls it and
+ * has no CPU fallback.
+ *
+ * Each function cites the reference lines it restates (paths relative to the
+ * reference tree).  The arithmetic of the sum lives in third-party HIP headers
+ * (operator+ of __half / __hip_bfloat16, ROCm 7.2 amd_hip_bf16.h:798-800,
+ * amd_hip_fp16.h:172-175): bf16 = fp32 add then round-to-nearest-even, fp16 =
+ * IEEE half add, fp32 = native add.  Everything here is integer bit work so the
+ * result does not depend on the host compiler's floating point options, except
+ * the single fp32 addition which is IEEE on x86-64 SSE (no flush-to-zero).
+ *
+ * Pinned by (see tests): torch-CPU adds, an exact rational-arithmetic brute
+ * force, exhaustive sweeps against numpy float16, a host compile of the HIP
+ * headers' own operator+, and committed golden vectors.
+ * Parity unpinned: NaN payload and sign of a NaN result (configs are finite).
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+#include <stdlib.h>
+#include <pthread.h>
+#include <time.h>
+
+/* ---------------------------------------------------------------- conversions */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* bf16 is the upper half of an fp32 word: widening is exact. */
+uint32_t orc_bf16_to_f32bits(uint16_t h) { return (uint32_t)h << 16; }
+
+/* fp32 -> bf16, round to nearest, ties to even.  NaN is quieted. */
+uint16_t orc_f32bits_to_bf16(uint32_t u)
+{
+    if ((u & 0x7fffffffu) > 0x7f800000u)          /* NaN: keep sign+top payload, force quiet bit */
+        return (uint16_t)((u >> 16) | 0x0040u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;                            /* carries into exponent; overflow lands on Inf */
+    return (uint16_t)(u >> 16);
+}
+
+/* fp16 -> fp32, exact (subnormals normalised). */
+uint32_t orc_f16_to_f32bits(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (exp == 0x1fu) return sign | 0x7f800000u | (man << 13);       /* Inf / NaN */
+    if (exp == 0) {
+        if (man == 0) return sign;                                   /* +-0 */
+        int e = -1;
+        do { man <<= 1; e++; } while (!(man & 0x400u));              /* normalise */
+        man &= 0x3ffu;
+        return sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+    }
+    return sign | ((exp + 127 - 15) << 23) | (man << 13);
+}
+
+/* fp32 -> fp16, round to nearest, ties to even; handles subnormal results and overflow. */
+uint16_t orc_f32bits_to_f16(uint32_t u)
+{
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu));  /* NaN, quiet */
+    if (a >= 0x477ff000u) {                       /* >= 65520 rounds to Inf (65504 is max finite) */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (a < 0x38800000u) {                        /* |x| < 2^-14 : subnormal half or zero */
+        if (a < 0x33000000u) return sign;         /* < 2^-25 : rounds to zero (2^-25 itself is a tie -> even = 0) */
+        uint32_t e = a >> 23;                     /* biased fp32 exponent, 102..112 */
+        uint32_t m = (a & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+        uint32_t shift = 126u - e;                /* result = m >> shift in units of 2^-24, shift 14..24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);              /* q may reach 0x400 = smallest normal: correct */
+    }
+    uint32_t e = (a >> 23) - 127 + 15;            /* 1..30 */
+    uint32_t m = a & 0x7fffffu;
+    uint32_t q = (e << 10) | (m >> 13);
+    uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;   /* carry may bump exponent, up to Inf */
+    return (uint16_t)(sign | q);
+}
+
+/* ---------------------------------------------------------------- the sum
+ * Restates k_acc<T> (step4/libtbvcoll.cpp:162-166): out[i] = a[i] + b[i] in T,
+ * where T's operator+ is the HIP header one (see file header).
+ * dtype codes as in step4/libtbvcoll.cpp:416 : 0=f32 1=f16 2=bf16.
+ * `out` may alias `a` (in-place, step4/libtbvcoll.cpp:421).
+ */
+static inline uint16_t sum_bf16(uint16_t a, uint16_t b)
+{
+    float s = u2f(orc_bf16_to_f32bits(a)) + u2f(orc_bf16_to_f32bits(b));
+    return orc_f32bits_to_bf16(f2u(s));
+}
+static inline uint16_t sum_f16(uint16_t a, uint16_t b)
+{
+    /* fp32 holds any sum of two halves exactly enough (24 >= 2*11+2): the
+     * second rounding is the only one that can be inexact. */
+    float s = u2f(orc_f16_to_f32bits(a)) + u2f(orc_f16_to_f32bits(b));
+    return orc_f32bits_to_f16(f2u(s));
+}
+
+uint16_t orc_sum1_bf16(uint16_t a, uint16_t b) { return sum_bf16(a, b); }
+uint16_t orc_sum1_f16(uint16_t a, uint16_t b) { return sum_f16(a, b); }
+
+static void sum_range(int dtype, const void* a, const void* b, void* out, size_t lo, size_t hi)
+{
+    if (dtype == 0) {
+        const float* x = (const float*)a; const float* y = (const float*)b; float* o = (float*)out;
+        for (size_t i = lo; i < hi; i++) o[i] = x[i] + y[i];
+    } else if (dtype == 1) {
+        const uint16_t* x = (const uint16_t*)a; const uint16_t* y = (const uint16_t*)b; uint16_t* o = (uint16_t*)out;
+        for (size_t i = lo; i < hi; i++) o[i] = sum_f16(x[i], y[i]);
+    } else {
+        const uint16_t* x = (const uint16_t*)a; const uint16_t* y = (const uint16_t*)b; uint16_t* o = (uint16_t*)out;
+        for (size_t i = lo; i < hi; i++) o[i] = sum_bf16(x[i], y[i]);
+    }
+}
+
+int orc_elem_size(int dtype) { return dtype == 0 ? 4 : 2; }
+
+/* n = element count (reference: m = nbytes / sizeof(T), step4/libtbvcoll.cpp:497-502;
+ * trailing bytes that do not fill an element are not summed). */
+int orc_sum(int dtype, const void* a, const void* b, void* out, size_t n)
+{
+    if (dtype < 0 || dtype > 2) return -1;
+    sum_range(dtype, a, b, out, 0, n);
+    return 0;
+}
+
+/* ---------------------------------------------------------------- the pack copy
+ * Restates the data movement of k_copy_sig (step4/libtbvcoll.cpp:131-134): byte
+ * identity src -> dst for n bytes (16-byte body + byte tail is an implementation
+ * detail), and, when tagging is on, the 64-bit sequence number stored at
+ * dst + align8(n) (step4/libtbvcoll.cpp:430,460).
+ */
+size_t orc_tag_offset(size_t nbytes) { return (nbytes + 7) & ~(size_t)7; }
+
+void orc_pack(void* dst, const void* src, size_t n, int tag, uint64_t seq)
+{
+    const unsigned char* s = (const unsigned char*)src;
+    unsigned char* d = (unsigned char*)dst;
+    for (size_t i = 0; i < n; i++) d[i] = s[i];
+    if (tag) memcpy(d + orc_tag_offset(n), &seq, 8);
+}
+
+/* ---------------------------------------------------------------- sizing / addressing
+ * step4/libtbvcoll.cpp:281 (cap rounded up to 4096), :297 (stride), :430 (xbytes),
+ * :431 (rail count), :436 (slot), :173-177 (rail fragment), :300-301 (send high-water mark),
+ * :287-288 (NSLOT clamp), :457 and :497 (launch shapes, informational).
+ */
+size_t orc_cap_round(size_t cap) { return (cap + 4095) & ~(size_t)4095; }
+size_t orc_stride(size_t cap_rounded, int tag) { return cap_rounded + (tag ? 4096 : 0); }
+size_t orc_xbytes(size_t nbytes, int tag) { return tag ? orc_tag_offset(nbytes) + 8 : nbytes; }
+int orc_rails_for(size_t nbytes, size_t rail1max, int nrails) { return nbytes <= rail1max ? 1 : nrails; }
+int orc_slot(uint64_t seq, int nslot) { return (int)(seq % (uint64_t)nslot); }
+int orc_nslot_clamp(int v) { if (v < 2) v = 2; if (v > 32) v = 32; return v; }
+
+/* returns 1 and fills off/len when rail `idx` of `R` owns bytes of an xbytes transfer, else 0 */
+int orc_fragment(size_t xbytes, int R, int idx, size_t* off, size_t* len)
+{
+    size_t chunk = ((xbytes / (size_t)R) + 4095) & ~(size_t)4095;
+    size_t roff = (size_t)idx * chunk;
+    if (roff >= xbytes) return 0;
+    size_t rlen = xbytes - roff; if (rlen > chunk) rlen = chunk;
+    if (off) *off = roff;
+    if (len) *len = rlen;
+    return 1;
+}
+
+int orc_wr_hwm(int nslot, size_t cap_rounded, size_t chunkb)
+{
+    size_t per_item = chunkb ? ((cap_rounded + chunkb - 1) / chunkb + 1) : 1;
+    size_t h = (size_t)(nslot - 1) * per_item; if (h > 96) h = 96;
+    int r = (int)h; if (r < 1) r = 1; return r;
+}
+
+int orc_pack_grid(size_t nbytes)
+{
+    size_t v = (nbytes + 15) / 16; size_t bl = (v + 255) / 256; if (bl > 320) bl = 320; if (bl < 1) bl = 1; return (int)bl;
+}
+int orc_sum_grid(size_t m) { size_t bl = (m + 255) / 256; if (bl > 160) bl = 160; return (int)bl; }
+
+/* log2 size bucket of the histogram, step4/libtbvcoll.cpp:208 */
+int orc_hist_bucket(size_t nbytes) { int b = 0; size_t v = nbytes; while (v >>= 1) b++; if (b > 31) b = 31; return b; }
+
+/* ---------------------------------------------------------------- ring / release model
+ * A host-only model of the slot ring and last-arriver release
+ * (step4/libtbvcoll.cpp:435-436,441-443,470-473,268-274).  Given a list of call
+ * sizes and an arrival script (sequence of rail ids; each rail consumes its own
+ * occurrences in FIFO order), it replays the protocol and writes, per arrival,
+ * the sequence number that got released (0 when the arrival was not the last
+ * rail of its call).  Returns the number of arrivals consumed, or a negative
+ * code when the script violates the protocol:
+ *   -1 a rail arrived with an empty queue, -2 ring overrun (depth > nslot).
+ */
+typedef struct { uint64_t seq; int slot; int R; } orc_item;
+
+long orc_ring_model(const size_t* call_nbytes, size_t ncalls, const int* script, size_t nscript,
+                    int nslot, int nrails, size_t rail1max, int depth,
+                    uint64_t* released /* [nscript] */, int* slots /* [ncalls] */, int* rails /* [ncalls] */)
+{
+    enum { MAXR = 4, MAXS = 32 };
+    orc_item q[MAXR][MAXS];
+    uint64_t head[MAXR] = {0}, tail[MAXR] = {0};
+    unsigned rails_done[MAXS] = {0};
+    uint64_t gflag[MAXS] = {0};
+    uint64_t seq = 0, done_upto = 0;
+    unsigned char rel_seen[64] = {0};          /* released-but-not-yet-retired marks, window <= nslot */
+    size_t next_call = 0, k = 0;
+    if (depth < 1) depth = 1;
+    if (depth > nslot) depth = nslot;
+    for (;;) {
+        /* caller: enqueue while it may run ahead: at most `depth` calls whose release is pending
+         * (a single stream cannot pack call s+depth before call s's wait has passed) */
+        while (next_call < ncalls && seq - done_upto < (uint64_t)depth) {
+            size_t nb = call_nbytes[next_call];
+            int R = orc_rails_for(nb, rail1max, nrails);
+            for (int r = 0; r < R; r++) if (head[r] - tail[r] >= (uint64_t)nslot) return -2;
+            seq++;
+            int slot = orc_slot(seq, nslot);
+            if (slots) slots[next_call] = slot;
+            if (rails) rails[next_call] = R;
+            for (int r = 0; r < R; r++) { orc_item it = { seq, slot, R }; q[r][head[r] % nslot] = it; head[r]++; }
+            next_call++;
+        }
+        if (k >= nscript) break;
+        int r = script[k];
+        if (r < 0 || r >= nrails || head[r] == tail[r]) return -1;
+        orc_item it = q[r][tail[r] % nslot];
+        uint64_t rel = 0;
+        if (++rails_done[it.slot] >= (unsigned)it.R) {
+            rails_done[it.slot] = 0; gflag[it.slot] = it.seq; rel = it.seq;
+            /* a 1-rail call may be released before an older 2-rail call; the stream
+             * retires waits in order, so only a contiguous prefix counts as done */
+            rel_seen[it.seq % 64] = 1;
+            while (rel_seen[(done_upto + 1) % 64]) { rel_seen[(done_upto + 1) % 64] = 0; done_upto++; }
+        }
+        tail[r]++;
+        if (released) released[k] = rel;
+        k++;
+    }
+    (void)gflag;
+    return (long)k;
+}
+
+/* ---------------------------------------------------------------- whole step, optionally threaded
+ * One all-reduce as the data path performs it: pack local -> bounce
+ * (step4/libtbvcoll.cpp:456-461), then out = local + received
+ * (step4/libtbvcoll.cpp:496-503).  Static contiguous partition over threads.
+ * Used as the host-core baseline by the bench and as a whole-step checker.
+ */
+typedef struct {
+    int dtype; const void* local; const void* peer; void* bounce; void* out; size_t lo, hi; size_t esz;
+} rc_job;
+
+static void* rc_worker(void* p)
+{
+    rc_job* j = (rc_job*)p;
+    if (j->bounce)
+        memcpy((char*)j->bounce + j->lo * j->esz, (const char*)j->local + j->lo * j->esz, (j->hi - j->lo) * j->esz);
+    sum_range(j->dtype, j->local, j->peer, j->out, j->lo, j->hi);
+    return NULL;
+}
+
+int orc_reduce_copy(int dtype, const void* local, const void* peer, void* bounce, void* out,
+                    size_t nbytes, int nthreads)
+{
+    if (dtype < 0 || dtype > 2) return -1;
+    size_t esz = (size_t)orc_elem_size(dtype), n = nbytes / esz;
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > 256) nthreads = 256;
+    if (nthreads == 1) {
+        rc_job j = { dtype, local, peer, bounce, out, 0, n, esz };
+        rc_worker(&j);
+        if (bounce && nbytes > n * esz) memcpy((char*)bounce + n * esz, (const char*)local + n * esz, nbytes - n * esz);
+        return 0;
+    }
+    pthread_t th[256]; rc_job jobs[256];
+    size_t per = (n + (size_t)nthreads - 1) / (size_t)nthreads;
+    per = (per + 63) & ~(size_t)63;
+    int started = 0;
+    for (int t = 0; t < nthreads; t++) {
+        size_t lo = (size_t)t * per, hi = lo + per; if (lo >= n) break; if (hi > n) hi = n;
+        rc_job j = { dtype, local, peer, bounce, out, lo, hi, esz }; jobs[t] = j;
+        if (pthread_create(&th[t], NULL, rc_worker, &jobs[t])) return -1;
+        started++;
+    }
+    for (int t = 0; t < started; t++) pthread_join(th[t], NULL);
+    if (bounce && nbytes > n * esz) memcpy((char*)bounce + n * esz, (const char*)local + n * esz, nbytes - n * esz);
+    return 0;
+}
+
+/* Median seconds per call of orc_reduce_copy over `reps` timed calls after `warm` untimed ones. */
+double orc_time_reduce_copy(int dtype, const void* local, const void* peer, void* bounce, void* out,
+                            size_t nbytes, int nthreads, int warm, int reps)
+{
+    if (reps < 1) reps = 1;
+    if (reps > 4096) reps = 4096;
+    double* t = (double*)malloc(sizeof(double) * (size_t)reps);
+    if (!t) return -1.0;
+    for (int i = 0; i < warm; i++) orc_reduce_copy(dtype, local, peer, bounce, out, nbytes, nthreads);
+    for (int i = 0; i < reps; i++) {
+        struct timespec a, b;
+        clock_gettime(CLOCK_MONOTONIC, &a);
+        orc_reduce_copy(dtype, local, peer, bounce, out, nbytes, nthreads);
+        clock_gettime(CLOCK_MONOTONIC, &b);
+        t[i] = (double)(b.tv_sec - a.tv_sec) + (double)(b.tv_nsec - a.tv_nsec) * 1e-9;
+    }
+    for (int i = 1; i < reps; i++) { double v = t[i]; int j = i - 1; while (j >= 0 && t[j] > v) { t[j + 1] = t[j]; j--; } t[j + 1] = v; }
+    double med = t[reps / 2];
+    free(t);
+    return med;
+}
