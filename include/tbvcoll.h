@@ -1,0 +1,168 @@
+/*
+ * tbvcoll.h -- C ABI of libtbvcoll.so, the MI355X (gfx950) build of the 2-rank
+ * tensor-parallel all-reduce data path.
+ *
+ * Part 1 is the drop-in boundary: the eleven symbols a caller of the reference
+ * library binds through ctypes (step4/tbvcoll.py:19-30), with the same argument
+ * meaning, return codes and threading rules.  Part 2 is additive: the emulated
+ * peer that stands in for everything that crossed a wire in the reference
+ * (step4/libtbvcoll.cpp:172-224,343-403), and a pipelined many-chunk entry point.
+ *
+ * Plain C types only.  Device pointers are raw HIP device addresses; `stream` is a
+ * raw hipStream_t.  The library never owns caller memory and touches caller
+ * buffers only from kernels launched on the caller's stream.
+ */
+#ifndef TBVCOLL_H
+#define TBVCOLL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ Part 1: drop-in boundary */
+
+/* dtype codes of tbv_ar_allreduce (step4/libtbvcoll.cpp:416). */
+#define TBV_DT_F32 0
+#define TBV_DT_F16 1
+#define TBV_DT_BF16 2
+
+/*
+ * Replaces tbv_ar_init (step4/libtbvcoll.cpp:279-414).
+ * rank: 0 or 1 (label only here).  devs: comma list naming the rails; only the
+ * count matters (1..4).  peer_ip/port: kept for signature parity, unused by the
+ * emulated peer.  cap: largest payload in bytes, rounded up to 4096.
+ * Reads TBV_ASYNC, TBV_GPUSIG, TBV_KWAIT, TBV_NSLOT, TBV_CHUNK, TBV_RAIL1MAX,
+ * TBV_CPU, TBV_WDOG, TBV_TAG, TBV_UNCACHED once.  Idempotent: a second call
+ * returns 0 and changes nothing.  Returns 0, or -1 after a "[tbvcoll] ..." line
+ * on stderr.
+ */
+int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_t cap);
+
+/*
+ * Replaces tbv_ar_allreduce (step4/libtbvcoll.cpp:417-508).
+ * out = ptr + peer, element-wise in `dtype`, for nbytes bytes; outp == NULL means
+ * in place.  Asynchronous: the result is valid in `stream` order.  Returns 0;
+ * -2 when nbytes exceeds the cap (caller falls back to its own collective);
+ * -1 when not initialised, after any earlier transfer error (sticky), or on a
+ * launch failure.  One caller thread at a time.
+ */
+int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype, void* stream);
+
+/* Replace tbv_ar_stats / tbv_ar_stats4 / tbv_ar_stats5 (step4/libtbvcoll.cpp:510-536):
+ * per-call averages in microseconds since the last read; any pointer may be NULL;
+ * reading resets. */
+void tbv_ar_stats(double* avg_us, unsigned long long* count);
+void tbv_ar_stats4(double* pre_us, double* xfer_us, double* post_us, double* enq_us,
+                   unsigned long long* count);
+void tbv_ar_stats5(double* pre_us, double* xfer_us, double* post_us, double* enq_us,
+                   double* drain_us, unsigned long long* count);
+
+/* Replace tbv_ar_cap / tbv_ar_async / tbv_ar_err (step4/libtbvcoll.cpp:537-539). */
+int tbv_ar_cap(void);
+int tbv_ar_async(void);
+int tbv_ar_err(void);
+
+/* Replace tbv_ar_rails / tbv_ar_hist (step4/libtbvcoll.cpp:542-561): dump per-rail
+ * and per-size transfer averages to stderr, then reset them. */
+void tbv_ar_rails(void);
+void tbv_ar_hist(void);
+
+/* Replaces tbv_ar_fini (step4/libtbvcoll.cpp:562-566): stops and joins the
+ * progress threads.  Frees nothing; the library stays initialised. */
+void tbv_ar_fini(void);
+
+/* ------------------------------------------------------------------ Part 2: emulated peer (additive)
+ *
+ * The reference's peer is a second machine reached through RDMA
+ * write-with-immediate (step4/libtbvcoll.cpp:181-203).  Here the peer is played
+ * on the same GPU: for every call, each rail's progress thread copies that
+ * rail's fragment of the peer payload into the receive slot on a side stream and
+ * then raises a 64-bit arrival word on that stream, which is the signal the
+ * immediate's completion gave.  None of these symbols exist in the reference.
+ */
+
+/* Queue the peer's payload for the next call that has none yet (FIFO, one entry per
+ * call).  `src` is a device pointer or pinned host memory holding at least the
+ * call's nbytes; it must stay valid until that call's result is complete.  Calls
+ * with no queued payload fall back to the repeat payload, then to mirror mode
+ * (the peer sends back this rank's own bounce slot, so out = 2 * in). */
+int tbv_emu_stage_peer(const void* src, size_t nbytes);
+
+/* Payload used by every call with an empty queue; NULL restores mirror mode. */
+int tbv_emu_stage_peer_repeat(const void* src, size_t nbytes);
+
+/* The peer ran ahead: copy `src` (nbytes <= cap) into every receive slot now and
+ * treat it as the already-arrived payload of each following call of at most
+ * nbytes that has no queued payload: such a call finds its flag up on entry, so
+ * its stream pays the pack, an already-satisfied wait and the sum.  Blocks until
+ * the copies are done.  src == NULL ends the mode. */
+int tbv_emu_peer_resident(const void* src, size_t nbytes);
+
+/* Arrival order: `rails[k]` is the rail whose fragment arrives k-th from now on.
+ * Each rail consumes its own occurrences in order and holds its signal until its
+ * turn (bounded by the watchdog).  n == 0 clears the script (free-running). */
+int tbv_emu_arrival_script(const int* rails, size_t n);
+
+/* Fault injection from the host: the peer never signals rail `rail` of call `seq`
+ * (seq counts calls from 1).  The watchdog must then trip.  seq == 0 clears. */
+int tbv_emu_withhold(unsigned long long seq, int rail);
+
+/* Sequence number of the last call issued (0 before the first). */
+unsigned long long tbv_emu_seq(void);
+
+/* Rail plan of a payload under the current settings: returns the rail count R and
+ * fills off[r], len[r] for r < R (len 0 when a rail owns nothing).  Pure host
+ * arithmetic; works without a GPU once TBV_* are read by tbv_emu_configure. */
+int tbv_emu_plan(size_t nbytes, size_t* off, size_t* len);
+
+/* Read the TBV_* environment and the rail count without touching the GPU, so the
+ * host logic (tbv_emu_plan, slot/cap arithmetic) can be exercised on a CPU box. */
+int tbv_emu_configure(const char* devs, size_t cap);
+
+/* Slot geometry and addresses (device pointers) for tests and benches. */
+int tbv_emu_nslot(void);
+size_t tbv_emu_stride(void);
+void* tbv_emu_send_slot(int slot);
+void* tbv_emu_recv_slot(int slot);
+
+/* Observed arrivals since the last read: fills up to `max` (seq, rail) pairs in
+ * the order the arrival words were seen; returns the count. */
+size_t tbv_emu_arrival_log(unsigned long long* seqs, int* rails, size_t max);
+
+/* Release-to-done latency probe.  When on, the sum kernel stores the call's seq
+ * to a host-visible word when its last block retires, and the progress thread
+ * that releases the GPU records (time it saw that word) - (time just before it
+ * raised the flag).  tbv_emu_latencies copies out up to `max` samples in
+ * microseconds and clears them. */
+int tbv_emu_latency_probe(int on);
+size_t tbv_emu_latencies(double* us, size_t max);
+
+/* Stale-data detector counters (TBV_TAG=1): checks, plain-load mismatches,
+ * system-scope-load mismatches. */
+void tbv_emu_tag_counts(unsigned long long* checks, unsigned long long* bad_plain,
+                        unsigned long long* bad_system);
+
+/* Full teardown so a process can re-initialise with other settings: joins threads,
+ * destroys streams, releases buffers (the uncached bounce slab is kept for reuse,
+ * never freed), clears the sticky error. */
+void tbv_emu_shutdown(void);
+
+/* Pipelined all-reduce of a payload larger than the cap: split into cap-sized
+ * chunks, each an ordinary call (own sequence number, slot and rail split), with
+ * up to NSLOT-1 chunks packed ahead so that the sum of chunk i overlaps the
+ * arrival of chunks i+1...  Queued peer payloads are consumed one per chunk.
+ * Same return codes as tbv_ar_allreduce, except that no size is over the cap. */
+int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, int dtype, void* stream);
+
+/* Standalone kernel entry points for benches and tests: run only the pack copy
+ * (into send slot `slot`, with completion signal) or only the sum, on `stream`. */
+int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream);
+int tbv_emu_run_sum(void* out, const void* a, const void* b, size_t nbytes, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TBVCOLL_H */

@@ -1,0 +1,59 @@
+// Internal interface between the host engine and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace tbv {
+
+// Footprint words the kernels leave in host-visible memory (same four the
+// reference keeps, step4/libtbvcoll.cpp:98): wait entered, wait passed, pack
+// started, sum done.
+enum Footprint { FP_WAIT_IN = 0, FP_WAIT_OUT = 1, FP_PACK = 2, FP_SUM_DONE = 3, FP_WAIT_TIMEOUT = 4 };
+
+struct PackArgs {
+    void* dst;                  // send slot (16-byte aligned)
+    const void* src;            // caller tensor
+    size_t nbytes;
+    unsigned long long* cflag;  // host-visible completion word of the slot
+    unsigned long long seq;
+    unsigned int* arrive;       // device counter of the slot, returns to 0
+    unsigned long long* tagp;   // where to store seq after the payload, or null
+    unsigned long long* fp;     // footprints or null
+};
+
+struct SumArgs {
+    void* out;
+    const void* a;              // caller tensor (may alias out)
+    const void* b;              // received payload
+    size_t nbytes;
+    int dtype;                  // 0 f32, 1 f16, 2 bf16
+    // optional in-kernel gate: block-leaders poll *wait_flag until >= seq
+    const unsigned long long* wait_flag;
+    unsigned long long seq;
+    unsigned long long spin_limit_ticks;   // bound of the in-kernel wait (100 MHz ticks)
+    // optional completion word (latency probe / footprint): last block stores seq
+    unsigned long long* done;
+    unsigned int* done_arrive;  // device counter, returns to 0
+    unsigned long long* fp;
+};
+
+// Launch geometry is exposed so the host can log and test it.
+int pack_grid(size_t nbytes);
+int sum_grid(size_t nbytes, int dtype);
+// Tuning knobs for experiments: vectors per lane per iteration (1,2,4,8) and the grid cap.
+void set_tuning(int unroll, int grid_cap);
+
+hipError_t launch_pack(const PackArgs& a, hipStream_t st);
+hipError_t launch_sum(const SumArgs& a, hipStream_t st);
+// One kernel that does pack (with completion signal) and sum: legal only when the
+// received payload is already in place.
+hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st);
+hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq,
+                           unsigned long long spin_limit_ticks, unsigned long long* fp, hipStream_t st);
+hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, unsigned long long* dbg,
+                         hipStream_t st);
+hipError_t launch_mark(unsigned long long* fp, int i, unsigned long long seq, hipStream_t st);
+hipError_t launch_fill_u32(unsigned int* p, unsigned int v, size_t n, hipStream_t st);
+
+}  // namespace tbv

@@ -1,0 +1,388 @@
+// gfx950 kernels of the all-reduce data path: the pack copy with its completion
+// signal, the two-operand sum, the fused pack+sum, and the small diagnostic
+// kernels.  Everything is elementwise and HBM-bound: 128-bit accesses, several
+// independent loads in flight per lane, no LDS, no MFMA.
+//
+// What each kernel replaces in the reference:
+//   k_step<.., PACK, ..>  k_copy_sig  step4/libtbvcoll.cpp:126-140
+//   k_step<.., SUM, ..>   k_acc<T>    step4/libtbvcoll.cpp:162-166
+//   k_waitflag            k_waitflag  step4/libtbvcoll.cpp:155-160
+//   k_tagchk / k_mark     k_tagchk / k_mark  step4/libtbvcoll.cpp:143-150,161
+#include <hip/hip_runtime.h>
+#include "tbv_kernels.h"
+
+namespace tbv {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+static constexpr int kThreads = 256;        // 4 wavefronts of 64
+static constexpr int kMaxSmallThreads = 1024;
+static constexpr int kMaxGrid = 256 * 8;     // 256 CUs, up to 8 resident blocks each
+
+// ---------------------------------------------------------------- arithmetic
+
+// bf16: widen both operands to fp32 (exact), add in fp32, round to nearest even.
+// The fptrunc of a float pair lowers to v_cvt_pk_bf16_f32 on gfx950.
+__device__ __forceinline__ uint32_t add_bf16x2(uint32_t x, uint32_t y)
+{
+    f32x2 s;
+    s.x = __uint_as_float(x << 16) + __uint_as_float(y << 16);
+    s.y = __uint_as_float(x & 0xffff0000u) + __uint_as_float(y & 0xffff0000u);
+    bf16x2 r = __builtin_convertvector(s, bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+template <int DT> __device__ __forceinline__ u32x4 add_vec(u32x4 x, u32x4 y);
+
+template <> __device__ __forceinline__ u32x4 add_vec<0>(u32x4 x, u32x4 y)
+{
+    f32x4 a = __builtin_bit_cast(f32x4, x), b = __builtin_bit_cast(f32x4, y);
+    f32x4 s;
+    s.x = a.x + b.x; s.y = a.y + b.y; s.z = a.z + b.z; s.w = a.w + b.w;
+    return __builtin_bit_cast(u32x4, s);
+}
+// fp16: the IEEE half add itself (what the HIP header's operator+ on _Float16 is);
+// it equals fp32-upcast + add + round-to-nearest-even for every finite pair.
+template <> __device__ __forceinline__ u32x4 add_vec<1>(u32x4 x, u32x4 y)
+{
+    f16x8 a = __builtin_bit_cast(f16x8, x), b = __builtin_bit_cast(f16x8, y);
+    f16x8 s = a + b;
+    return __builtin_bit_cast(u32x4, s);
+}
+template <> __device__ __forceinline__ u32x4 add_vec<2>(u32x4 x, u32x4 y)
+{
+    u32x4 r;
+    r.x = add_bf16x2(x.x, y.x); r.y = add_bf16x2(x.y, y.y);
+    r.z = add_bf16x2(x.z, y.z); r.w = add_bf16x2(x.w, y.w);
+    return r;
+}
+
+template <int DT> struct Elem;
+template <> struct Elem<0> { typedef float T; static __device__ __forceinline__ T add(T a, T b) { return a + b; } };
+template <> struct Elem<1> { typedef _Float16 T; static __device__ __forceinline__ T add(T a, T b) { return a + b; } };
+template <> struct Elem<2> {
+    typedef uint16_t T;
+    static __device__ __forceinline__ T add(T a, T b)
+    {
+        float s = __uint_as_float((uint32_t)a << 16) + __uint_as_float((uint32_t)b << 16);
+        __bf16 r = (__bf16)s;
+        return __builtin_bit_cast(uint16_t, r);
+    }
+};
+
+// ---------------------------------------------------------------- signalling helpers
+
+__device__ __forceinline__ void store_sys(unsigned long long* p, unsigned long long v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Every thread of the block calls this after its last store.  When the last
+// block of the grid gets here, all stores of the whole grid are visible system
+// wide and `word` is set to `seq`.  `arrive` counts blocks and returns to 0.
+__device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
+                                              unsigned int* arrive, unsigned int nblk)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");       // this wave's stores: performed, written back system wide
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        bool last = true;
+        if (nblk > 1) {
+            unsigned int prev = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            last = (prev == nblk - 1);
+            if (last) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (last) store_sys(word, seq);
+    }
+}
+
+// Block leader polls a host-visible word until it reaches seq, bounded by a tick
+// count of the 100 MHz constant clock so that every wave leaves the kernel even
+// if nobody ever raises the word.
+__device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsigned long long seq,
+                                          unsigned long long limit, unsigned long long* fp)
+{
+    if (threadIdx.x == 0) {
+        if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_IN, seq);
+        unsigned long long t0 = wall_clock64();
+        while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
+            __builtin_amdgcn_s_sleep(1);
+            if (wall_clock64() - t0 > limit) {
+                if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
+                break;
+            }
+        }
+        if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_OUT, seq);
+    }
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");       // payload written before the flag is visible to all waves
+}
+
+// ---------------------------------------------------------------- the step kernel
+//
+// One body for pack-only, sum-only and pack+sum.  Work unit = one 16-byte vector
+// per lane; a block covers blockDim*U consecutive vectors per iteration with the
+// U loads of a lane blockDim vectors apart, so each wavefront instruction touches
+// 1 KiB of consecutive memory and a lane has U (x2 for the sum) loads in flight.
+
+struct StepArgs {
+    // pack
+    u32x4* bounce; unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long* tagp;
+    // sum
+    u32x4* out; const u32x4* b;
+    const unsigned long long* wait_flag; unsigned long long spin_limit;
+    unsigned long long* done; unsigned int* done_arrive;
+    // common
+    const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp;
+};
+
+template <int DT, int U, bool PACK, bool SUM>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
+{
+    const unsigned tid = threadIdx.x, nthr = blockDim.x;
+    if (PACK && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.fp);
+
+    const size_t nvec = g.nbytes >> 4;
+    const size_t tile = (size_t)nthr * U;
+    for (size_t base = (size_t)blockIdx.x * tile; base < nvec; base += (size_t)gridDim.x * tile) {
+        u32x4 x[U], y[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            size_t i = base + (size_t)u * nthr + tid;
+            if (i < nvec) {
+                x[u] = g.a[i];
+                if (SUM) y[u] = __builtin_nontemporal_load(g.b + i);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            size_t i = base + (size_t)u * nthr + tid;
+            if (i < nvec) {
+                if (PACK) g.bounce[i] = x[u];
+                if (SUM) g.out[i] = add_vec<DT>(x[u], y[u]);
+            }
+        }
+    }
+    // bytes past the last whole vector
+    const unsigned tail = (unsigned)(g.nbytes & 15);
+    if (tail && blockIdx.x == 0) {
+        const size_t off = nvec << 4;
+        if (PACK && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
+        if (SUM) {
+            typedef typename Elem<DT>::T T;
+            const unsigned ne = tail / sizeof(T);
+            if (tid < ne) {
+                const T* pa = (const T*)((const char*)g.a + off);
+                const T* pb = (const T*)((const char*)g.b + off);
+                T* po = (T*)((char*)g.out + off);
+                po[tid] = Elem<DT>::add(pa[tid], pb[tid]);
+            }
+        }
+    }
+    if (PACK) {
+        if (g.tagp && blockIdx.x == 0 && tid == 0) *g.tagp = g.seq;
+        grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x);
+    }
+    if (SUM && g.done) {
+        grid_complete(g.done, g.seq, g.done_arrive, gridDim.x);
+    }
+}
+
+// Fallback bodies for caller pointers that are not 16-byte aligned: element (sum)
+// or 4/1-byte (pack) grid-stride loops.  Same results, lower bandwidth.
+template <typename W>
+__global__ __launch_bounds__(kThreads) void k_pack_narrow(PackArgs a)
+{
+    if (a.fp && blockIdx.x == 0 && threadIdx.x == 0) store_sys(a.fp + FP_PACK, a.seq);
+    const size_t n = a.nbytes / sizeof(W);
+    const W* s = (const W*)a.src; W* d = (W*)a.dst;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) d[i] = s[i];
+    const unsigned tail = (unsigned)(a.nbytes - n * sizeof(W));
+    if (blockIdx.x == 0 && threadIdx.x < tail)
+        ((unsigned char*)a.dst)[n * sizeof(W) + threadIdx.x] = ((const unsigned char*)a.src)[n * sizeof(W) + threadIdx.x];
+    if (a.tagp && blockIdx.x == 0 && threadIdx.x == 0) *a.tagp = a.seq;
+    grid_complete(a.cflag, a.seq, a.arrive, gridDim.x);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void k_sum_narrow(SumArgs a)
+{
+    typedef typename Elem<DT>::T T;
+    if (a.wait_flag) gate_wait(a.wait_flag, a.seq, a.spin_limit_ticks, a.fp);
+    const size_t n = a.nbytes / sizeof(T);
+    const T* x = (const T*)a.a; const T* y = (const T*)a.b; T* o = (T*)a.out;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        o[i] = Elem<DT>::add(x[i], y[i]);
+    if (a.done) grid_complete(a.done, a.seq, a.done_arrive, gridDim.x);
+}
+
+// ---------------------------------------------------------------- diagnostics
+
+__global__ void k_waitflag(const unsigned long long* flag, unsigned long long seq, unsigned long long limit,
+                           unsigned long long* fp)
+{
+    gate_wait(flag, seq, limit, fp);
+}
+
+// Re-reads the sequence tag the pack kernel appended to the payload, once with a
+// plain load and once with a system-scope load, and counts disagreements.
+// dbg: [checks, plain mismatches, system mismatches, first bad seq, first plain value, first system value]
+__global__ void k_tagchk(const unsigned long long* tag, unsigned long long seq, unsigned long long* dbg)
+{
+    unsigned long long v1 = *(const volatile unsigned long long*)tag;
+    unsigned long long v2 = __hip_atomic_load(tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_fetch_add(dbg + 0, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (v1 != seq) __hip_atomic_fetch_add(dbg + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (v2 != seq) __hip_atomic_fetch_add(dbg + 2, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if ((v1 != seq || v2 != seq) && dbg[3] == 0) { dbg[3] = seq; dbg[4] = v1; dbg[5] = v2; }
+}
+
+__global__ void k_mark(unsigned long long* fp, int i, unsigned long long seq) { store_sys(fp + i, seq); }
+
+__global__ void k_fill_u32(unsigned int* p, unsigned int v, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// ---------------------------------------------------------------- launch geometry
+
+static int g_unroll = 4;        // vectors per lane per iteration for the large path
+static int g_grid_cap = kMaxGrid;
+
+struct Geom { int grid, block, unroll; };
+
+static Geom geom_for(size_t nbytes)
+{
+    size_t nvec = nbytes >> 4;
+    Geom g;
+    if (nvec <= (size_t)kMaxSmallThreads) {
+        // one block, one vector per lane: no cross-block arrival counting on the latency path
+        int thr = (int)((nvec + 63) / 64 * 64);
+        if (thr < 64) thr = 64;
+        g.grid = 1; g.block = thr; g.unroll = 1;
+        return g;
+    }
+    g.block = kThreads;
+    g.unroll = (nvec >= (size_t)kThreads * 16) ? g_unroll : 1;
+    size_t tile = (size_t)g.block * g.unroll;
+    size_t tiles = (nvec + tile - 1) / tile;
+    g.grid = (int)(tiles < (size_t)g_grid_cap ? tiles : (size_t)g_grid_cap);
+    if (g.grid < 1) g.grid = 1;
+    return g;
+}
+
+int pack_grid(size_t nbytes) { return geom_for(nbytes).grid; }
+int sum_grid(size_t nbytes, int) { return geom_for(nbytes).grid; }
+
+void set_tuning(int unroll, int grid_cap)
+{
+    if (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) g_unroll = unroll;
+    if (grid_cap >= 1 && grid_cap <= 65535) g_grid_cap = grid_cap;
+}
+
+static inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+template <int DT, bool PACK, bool SUM>
+static hipError_t launch_step_u(const StepArgs& s, const Geom& g, hipStream_t st)
+{
+    switch (g.unroll) {
+        case 1: hipLaunchKernelGGL((k_step<DT, 1, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
+        case 2: hipLaunchKernelGGL((k_step<DT, 2, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
+        case 8: hipLaunchKernelGGL((k_step<DT, 8, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
+        default: hipLaunchKernelGGL((k_step<DT, 4, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
+    }
+    return hipGetLastError();
+}
+
+template <bool PACK, bool SUM>
+static hipError_t launch_step(int dtype, const StepArgs& s, const Geom& g, hipStream_t st)
+{
+    if (!SUM) return launch_step_u<0, PACK, SUM>(s, g, st);      // the copy does not depend on the element type
+    switch (dtype) {
+        case 0: return launch_step_u<0, PACK, SUM>(s, g, st);
+        case 1: return launch_step_u<1, PACK, SUM>(s, g, st);
+        case 2: return launch_step_u<2, PACK, SUM>(s, g, st);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_pack(const PackArgs& a, hipStream_t st)
+{
+    if (!a.dst || !a.src || !a.cflag || !a.arrive || !al16(a.dst)) return hipErrorInvalidValue;
+    if (al16(a.src)) {
+        StepArgs s{};
+        s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive; s.tagp = a.tagp;
+        s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
+        return launch_step<true, false>(0, s, geom_for(a.nbytes), st);
+    }
+    size_t units = a.nbytes / 4 + 1;
+    int grid = (int)((units + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid;
+    if ((((uintptr_t)a.src) & 3) == 0) hipLaunchKernelGGL((k_pack_narrow<uint32_t>), dim3(grid), dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((k_pack_narrow<unsigned char>), dim3(grid), dim3(kThreads), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_sum(const SumArgs& a, hipStream_t st)
+{
+    if (!a.out || !a.a || !a.b || a.dtype < 0 || a.dtype > 2) return hipErrorInvalidValue;
+    if (a.done && !a.done_arrive) return hipErrorInvalidValue;
+    if (al16(a.out) && al16(a.a) && al16(a.b)) {
+        StepArgs s{};
+        s.out = (u32x4*)a.out; s.b = (const u32x4*)a.b; s.wait_flag = a.wait_flag; s.spin_limit = a.spin_limit_ticks;
+        s.done = a.done; s.done_arrive = a.done_arrive;
+        s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
+        return launch_step<false, true>(a.dtype, s, geom_for(a.nbytes), st);
+    }
+    size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
+    int grid = (int)((n + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid; if (grid < 1) grid = 1;
+    switch (a.dtype) {
+        case 0: hipLaunchKernelGGL((k_sum_narrow<0>), dim3(grid), dim3(kThreads), 0, st, a); break;
+        case 1: hipLaunchKernelGGL((k_sum_narrow<1>), dim3(grid), dim3(kThreads), 0, st, a); break;
+        default: hipLaunchKernelGGL((k_sum_narrow<2>), dim3(grid), dim3(kThreads), 0, st, a); break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st)
+{
+    if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes)
+        return hipErrorInvalidValue;
+    if (q.done && !q.done_arrive) return hipErrorInvalidValue;
+    if (q.wait_flag) return hipErrorInvalidValue;     // waiting for the peer before sending to it would deadlock two real ranks
+    StepArgs s{};
+    s.bounce = (u32x4*)p.dst; s.cflag = p.cflag; s.pack_arrive = p.arrive; s.tagp = p.tagp;
+    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.spin_limit = q.spin_limit_ticks;
+    s.done = q.done; s.done_arrive = q.done_arrive;
+    s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp;
+    return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes), st);
+}
+
+hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq, unsigned long long limit,
+                           unsigned long long* fp, hipStream_t st)
+{
+    hipLaunchKernelGGL(k_waitflag, dim3(1), dim3(64), 0, st, flag, seq, limit, fp);
+    return hipGetLastError();
+}
+hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, unsigned long long* dbg, hipStream_t st)
+{
+    hipLaunchKernelGGL(k_tagchk, dim3(1), dim3(1), 0, st, tag, seq, dbg);
+    return hipGetLastError();
+}
+hipError_t launch_mark(unsigned long long* fp, int i, unsigned long long seq, hipStream_t st)
+{
+    hipLaunchKernelGGL(k_mark, dim3(1), dim3(1), 0, st, fp, i, seq);
+    return hipGetLastError();
+}
+hipError_t launch_fill_u32(unsigned int* p, unsigned int v, size_t n, hipStream_t st)
+{
+    int grid = (int)((n + kThreads - 1) / kThreads); if (grid < 1) grid = 1; if (grid > 1024) grid = 1024;
+    hipLaunchKernelGGL(k_fill_u32, dim3(grid), dim3(kThreads), 0, st, p, v, n);
+    return hipGetLastError();
+}
+
+}  // namespace tbv
