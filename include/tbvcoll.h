@@ -140,6 +140,13 @@ size_t tbv_emu_arrival_log(unsigned long long* seqs, int* rails, size_t max);
 int tbv_emu_latency_probe(int on);
 size_t tbv_emu_latencies(double* us, size_t max);
 
+/* Per-kernel timing: when on, every pack launch (which = 0) and every sum or
+ * pack+sum launch (which = 1) is bracketed by two events on the caller's stream.
+ * tbv_emu_kernel_times synchronises the device, returns the number of recorded
+ * launches and their mean and minimum duration in microseconds, then forgets them. */
+int tbv_emu_kernel_timing(int on);
+size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_us);
+
 /* Stale-data detector counters (TBV_TAG=1): checks, plain-load mismatches,
  * system-scope-load mismatches. */
 void tbv_emu_tag_counts(unsigned long long* checks, unsigned long long* bad_plain,

@@ -80,7 +80,7 @@ struct Staged { const char* ptr; size_t nbytes; };
 struct Engine {
     // configuration
     int configured = 0, inited = 0, rank = 0, R = 0, async = 1, nslot = 8, gpusig = 1, kwait = 0;
-    int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0;
+    int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     size_t cap = 0, stride = 0, rail1max = 96u * 1024u, chunkb = 0, fusewait_max = 0;
     double wdog = 10.0;
     int can_wait_value = 1, can_write_value = 1;
@@ -88,7 +88,7 @@ struct Engine {
     char* sendbase = nullptr;
     char* recvbase = nullptr;
     char* hostwords = nullptr;                // one coherent host block holding every flag word
-    unsigned int* counters = nullptr;         // device: arrive[MAXSLOT], done_arrive[MAXSLOT]
+    unsigned int* counters = nullptr;         // device: per slot one counter block for the pack, one for the sum
     hipEvent_t ev[MAXSLOT] = {};
     // protocol state
     Rail rr[MAXRAIL];
@@ -115,6 +115,10 @@ struct Engine {
     std::vector<std::pair<uint64_t, int>> arrivals;
     std::atomic<int> probe{0};
     std::vector<double> latencies;
+    // optional per-kernel timing with events on the caller's stream: [0]=pack, [1]=sum
+    int ktime = 0;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> kev[2];
+    size_t kev_used[2] = {0, 0};
     // statistics (guarded by smx)
     std::mutex smx;
     double t_acc = 0, t_pre = 0, t_post = 0, t_enq = 0, t_drain = 0;
@@ -149,6 +153,9 @@ inline unsigned long long* scratchword() { return word(W_MISC, 4); }
 inline uint64_t ld_acq(const unsigned long long* p) { return __atomic_load_n(p, __ATOMIC_ACQUIRE); }
 inline void st_rel(unsigned long long* p, uint64_t v) { __atomic_store_n(p, (unsigned long long)v, __ATOMIC_RELEASE); }
 
+inline unsigned int* pack_counters(int s) { return G.counters + (size_t)s * tbv::kCounterWords; }
+inline unsigned long long* relay_word(int s) { return (unsigned long long*)(G.counters + (size_t)2 * MAXSLOT * tbv::kCounterWords) + (size_t)s * 8; }
+inline unsigned int* done_counters(int s) { return G.counters + (size_t)(MAXSLOT + s) * tbv::kCounterWords; }
 inline char* slot_send(int s) { return G.sendbase + (size_t)s * G.stride; }
 inline char* slot_recv(int s) { return G.recvbase + (size_t)s * G.stride; }
 inline size_t tag_offset(size_t nbytes) { return (nbytes + 7) & ~(size_t)7; }
@@ -370,6 +377,8 @@ int configure(const char* devs, size_t cap)
     G.uncached = geti("TBV_UNCACHED", 1);
     G.railsum = geti("TBV_RAILSUM", 0);
     G.fuse = geti("TBV_FUSE", 0);
+    // uncached bounce: waves only drain their stores; cached bounce: block leader writes the L2 back
+    G.packsig = geti("TBV_PACKSIG", (G.uncached & 1) ? 0 : 1);
     G.fusewait_max = getz("TBV_FUSEWAIT", 0);
     G.stride = G.cap + (G.tag ? 4096 : 0);
     { size_t per_item = G.chunkb ? ((G.cap + G.chunkb - 1) / G.chunkb + 1) : 1;
@@ -398,6 +407,28 @@ void free_slab(char* p, const SlabCache& cache)
 }
 
 // ---- enqueue halves --------------------------------------------------------------------
+
+// Event pair for one kernel launch when kernel timing is on (pool grows on demand).
+// The events are handed to the launch itself, so they carry that dispatch's own
+// start and end timestamps.
+struct KTimer {
+    tbv::Timing t;
+    bool on;
+    explicit KTimer(int which) : on(G.ktime != 0)
+    {
+        if (!on) return;
+        auto& pool = G.kev[which];
+        if (G.kev_used[which] == pool.size()) {
+            hipEvent_t a, b;
+            if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { on = false; return; }
+            pool.emplace_back(a, b);
+        }
+        t.start = pool[G.kev_used[which]].first;
+        t.stop = pool[G.kev_used[which]].second;
+        G.kev_used[which]++;
+    }
+    const tbv::Timing* get() const { return on ? &t : nullptr; }
+};
 
 struct Call {
     uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused;
@@ -448,9 +479,10 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
 
     tbv::PackArgs pa{};
     pa.dst = slot_send(c->slot); pa.src = ptr; pa.nbytes = nbytes;
-    pa.cflag = cflag(c->slot); pa.seq = c->seq; pa.arrive = G.counters + c->slot;
+    pa.cflag = cflag(c->slot); pa.seq = c->seq; pa.arrive = pack_counters(c->slot);
     pa.tagp = G.tag ? (unsigned long long*)(slot_send(c->slot) + tagoff) : nullptr;
     pa.fp = G.kwait ? footprints() : nullptr;
+    pa.sigmode = G.packsig;
 
     if (G.async) {
         // An early flag must not release an older call of this slot that some rail has not finished:
@@ -463,10 +495,14 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             if (can_fuse) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
-                if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = G.counters + MAXSLOT + c->slot; }
-                if (tbv::launch_pack_sum(pa, sa, st) != hipSuccess) FAIL("pack+sum kernel launch failed");
+                if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
+                KTimer kt(1);
+                if (tbv::launch_pack_sum(pa, sa, st, kt.get()) != hipSuccess) FAIL("pack+sum kernel launch failed");
                 c->fused = true;
-            } else if (tbv::launch_pack(pa, st) != hipSuccess) FAIL("pack kernel launch failed");
+            } else {
+                KTimer kt(0);
+                if (tbv::launch_pack(pa, st, kt.get()) != hipSuccess) FAIL("pack kernel launch failed");
+            }
         } else {
             if (hipMemcpyAsync(slot_send(c->slot), ptr, nbytes, hipMemcpyDeviceToDevice, st) != hipSuccess) FAIL("copy into send slot failed");
             if (hipEventRecord(G.ev[c->slot], st) != hipSuccess) FAIL("event record failed");
@@ -511,10 +547,11 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         tbv::SumArgs sa{};
         sa.out = (char*)outp + off; sa.a = (const char*)ptr + off; sa.b = rb + off;
         sa.nbytes = len; sa.dtype = dtype; sa.seq = c.seq;
-        sa.wait_flag = gate; sa.spin_limit_ticks = spin_ticks;
+        sa.wait_flag = gate; sa.relay = gate ? relay_word(c.slot) : nullptr; sa.spin_limit_ticks = spin_ticks;
         sa.fp = G.kwait ? footprints() : nullptr;
-        if (probe && last) { sa.done = doneword(c.slot); sa.done_arrive = G.counters + MAXSLOT + c.slot; }
-        if (tbv::launch_sum(sa, st) != hipSuccess) FAIL("sum kernel launch failed");
+        if (probe && last) { sa.done = doneword(c.slot); sa.done_arrive = done_counters(c.slot); }
+        KTimer kt(1);
+        if (tbv::launch_sum(sa, st, kt.get()) != hipSuccess) FAIL("sum kernel launch failed");
         return 0;
     };
     auto gate_stream = [&](unsigned long long* flag) -> int {
@@ -541,8 +578,11 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
             if (sum_piece(off, l, nullptr, pieces == total) != 0) return -1;
         }
     } else {
-        const bool fusewait = G.async && c.nbytes <= G.fusewait_max && !G.tag && G.kwait != 1;
-        if (G.async && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
+        // The flag may already be up when the call is made (the peer was early): the payload is then in
+        // place before the sum is even launched and the stream needs no gate at all.
+        const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
+        const bool fusewait = G.async && !arrived && c.nbytes <= G.fusewait_max && !G.tag && G.kwait != 1;
+        if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
             if (tbv::launch_tagchk((const unsigned long long*)(rb + tag_offset(c.nbytes)), c.seq, dbgwords(), st) != hipSuccess)
                 FAIL("tag check launch failed");
@@ -608,8 +648,9 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     const size_t wbytes = (size_t)W_BLOCKS * MAXSLOT * FLAG_STRIDE;
     if (hipHostMalloc((void**)&G.hostwords, wbytes, hipHostMallocCoherent) != hipSuccess) FAIL("host flag block allocation failed");
     memset(G.hostwords, 0, wbytes);
-    if (hipMalloc((void**)&G.counters, sizeof(unsigned int) * 2 * MAXSLOT) != hipSuccess) FAIL("counter allocation failed");
-    if (hipMemset(G.counters, 0, sizeof(unsigned int) * 2 * MAXSLOT) != hipSuccess) FAIL("counter clear failed");
+    const size_t cbytes = sizeof(unsigned int) * 2 * MAXSLOT * tbv::kCounterWords + (size_t)MAXSLOT * 64;
+    if (hipMalloc((void**)&G.counters, cbytes) != hipSuccess) FAIL("counter allocation failed");
+    if (hipMemset(G.counters, 0, cbytes) != hipSuccess) FAIL("counter clear failed");
     for (int i = 0; i < G.nslot; i++) {
         if (hipEventCreateWithFlags(&G.ev[i], hipEventReleaseToSystem | hipEventDisableTiming) != hipSuccess) {
             (void)hipGetLastError();
@@ -847,6 +888,34 @@ extern "C" size_t tbv_emu_latencies(double* us, size_t max)
     return n;
 }
 
+// Per-kernel timing with events recorded on the caller's stream right before and
+// after each pack (which 0) and sum / pack+sum (which 1) launch.
+extern "C" int tbv_emu_kernel_timing(int on)
+{
+    if (!G.inited) return -1;
+    G.ktime = on ? 1 : 0;
+    return 0;
+}
+
+// Mean, minimum and count of the recorded launches of one kernel; synchronises the
+// device, then forgets the samples.  Returns the count.
+extern "C" size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_us)
+{
+    if (!G.inited || which < 0 || which > 1) return 0;
+    (void)hipDeviceSynchronize();
+    double sum = 0, mn = 1e30;
+    size_t n = 0;
+    for (size_t i = 0; i < G.kev_used[which]; i++) {
+        float ms = 0;
+        if (hipEventElapsedTime(&ms, G.kev[which][i].first, G.kev[which][i].second) != hipSuccess) continue;
+        sum += ms * 1e3; mn = std::min(mn, (double)ms * 1e3); n++;
+    }
+    G.kev_used[which] = 0;
+    if (mean_us) *mean_us = n ? sum / (double)n : 0.0;
+    if (min_us) *min_us = n ? mn : 0.0;
+    return n;
+}
+
 extern "C" void tbv_emu_tag_counts(unsigned long long* checks, unsigned long long* bad_plain, unsigned long long* bad_system)
 {
     unsigned long long z[3] = {0, 0, 0};
@@ -868,6 +937,11 @@ extern "C" void tbv_emu_shutdown(void)
     free_slab(G.recvbase, g_uc_recv); G.recvbase = nullptr;
     if (G.hostwords) { (void)hipHostFree(G.hostwords); G.hostwords = nullptr; }
     if (G.counters) { (void)hipFree(G.counters); G.counters = nullptr; }
+    for (int w = 0; w < 2; w++) {
+        for (auto& p : G.kev[w]) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
+        G.kev[w].clear(); G.kev_used[w] = 0;
+    }
+    G.ktime = 0;
     G.staged.clear(); G.repeat = Staged{nullptr, 0}; G.resident_bytes = 0;
     G.script.clear(); G.turn.store(0); G.withhold_seq.store(0);
     { std::lock_guard<std::mutex> lk(G.logmx); G.arrivals.clear(); G.latencies.clear(); }
@@ -921,7 +995,7 @@ extern "C" int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* 
     tbv::PackArgs pa{};
     pa.dst = slot_send(slot); pa.src = src; pa.nbytes = nbytes;
     pa.cflag = word(W_MISC, 8 + slot % 16);          // a completion word nobody waits on
-    pa.seq = 1; pa.arrive = G.counters + slot;
+    pa.seq = 1; pa.arrive = pack_counters(slot); pa.sigmode = G.packsig;
     return tbv::launch_pack(pa, (hipStream_t)stream) == hipSuccess ? 0 : -1;
 }
 

@@ -17,9 +17,10 @@ struct PackArgs {
     size_t nbytes;
     unsigned long long* cflag;  // host-visible completion word of the slot
     unsigned long long seq;
-    unsigned int* arrive;       // device counter of the slot, returns to 0
+    unsigned int* arrive;       // the slot's counter lines (kCounterWords words), all return to 0
     unsigned long long* tagp;   // where to store seq after the payload, or null
     unsigned long long* fp;     // footprints or null
+    int sigmode;                // how block stores are made visible before the block is counted (see grid_complete)
 };
 
 struct SumArgs {
@@ -30,13 +31,21 @@ struct SumArgs {
     int dtype;                  // 0 f32, 1 f16, 2 bf16
     // optional in-kernel gate: block-leaders poll *wait_flag until >= seq
     const unsigned long long* wait_flag;
+    unsigned long long* relay;  // device word: block 0 polls wait_flag and republishes it here for the other blocks
     unsigned long long seq;
     unsigned long long spin_limit_ticks;   // bound of the in-kernel wait (100 MHz ticks)
     // optional completion word (latency probe / footprint): last block stores seq
     unsigned long long* done;
-    unsigned int* done_arrive;  // device counter, returns to 0
+    unsigned int* done_arrive;  // counter lines (kCounterWords words), all return to 0
     unsigned long long* fp;
 };
+
+// Optional exact timing of one launch: the two events receive the start and end
+// timestamps of that dispatch itself (hipExtLaunchKernel), not of the gaps around it.
+struct Timing { hipEvent_t start = nullptr, stop = nullptr; };
+
+// Words of device memory one grid-completion counter block needs (top line + group lines).
+static constexpr size_t kCounterWords = 16 * 128;
 
 // Launch geometry is exposed so the host can log and test it.
 int pack_grid(size_t nbytes);
@@ -44,11 +53,11 @@ int sum_grid(size_t nbytes, int dtype);
 // Tuning knobs for experiments: vectors per lane per iteration (1,2,4,8) and the grid cap.
 void set_tuning(int unroll, int grid_cap);
 
-hipError_t launch_pack(const PackArgs& a, hipStream_t st);
-hipError_t launch_sum(const SumArgs& a, hipStream_t st);
+hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t = nullptr);
+hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullptr);
 // One kernel that does pack (with completion signal) and sum: legal only when the
 // received payload is already in place.
-hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st);
+hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq,
                            unsigned long long spin_limit_ticks, unsigned long long* fp, hipStream_t st);
 hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, unsigned long long* dbg,

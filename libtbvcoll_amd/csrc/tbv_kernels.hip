@@ -9,6 +9,7 @@
 //   k_waitflag            k_waitflag  step4/libtbvcoll.cpp:155-160
 //   k_tagchk / k_mark     k_tagchk / k_mark  step4/libtbvcoll.cpp:143-150,161
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include "tbv_kernels.h"
 
 namespace tbv {
@@ -83,43 +84,83 @@ __device__ __forceinline__ void store_sys(unsigned long long* p, unsigned long l
 
 // Every thread of the block calls this after its last store.  When the last
 // block of the grid gets here, all stores of the whole grid are visible system
-// wide and `word` is set to `seq`.  `arrive` counts blocks and returns to 0.
+// wide and `word` is set to `seq`.
+//
+// Blocks are counted in two levels so that no single address takes one atomic
+// per block (same-address atomics retire one at a time): groups of kGroup blocks
+// count on their own 64-byte line, and the last block of a group counts on the
+// top line.  `ctr` points to the slot's counter lines (line 0 = top, line 1+g =
+// group g, 16 words apart); every counter is put back to 0 by its last arriver.
+//
+// mode 0: the destination is uncached memory: stores bypass the L2, so each wave
+//         only has to see its own stores acknowledged before the block is counted.
+//         (The workgroup-scope release inside __syncthreads does not wait for the
+//         store counter on gfx950, hence the explicit wait.)
+// mode 1: the destination may be cached: the block leader also writes the L2 back
+//         system wide after the barrier (one write-back per block).
+// mode 2: every wave writes back system wide before the barrier (most conservative).
+static constexpr unsigned kGroup = 32;
+static constexpr unsigned kCtrLine = 16;       // words per counter line (64 bytes)
+
 __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
-                                              unsigned int* arrive, unsigned int nblk)
+                                              unsigned int* ctr, unsigned int nblk, int mode)
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");       // this wave's stores: performed, written back system wide
+    if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
+        if (mode == 1) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
         bool last = true;
         if (nblk > 1) {
-            unsigned int prev = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            last = (prev == nblk - 1);
-            if (last) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned g = blockIdx.x / kGroup, ngroups = (nblk + kGroup - 1) / kGroup;
+            const unsigned pop = min(kGroup, nblk - g * kGroup);
+            unsigned int* gc = ctr + kCtrLine * (1 + g);
+            last = false;
+            if (__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == pop - 1) {
+                __hip_atomic_store(gc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (ngroups == 1) last = true;
+                else if (__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1) {
+                    __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = true;
+                }
+            }
         }
         if (last) store_sys(word, seq);
     }
 }
 
-// Block leader polls a host-visible word until it reaches seq, bounded by a tick
-// count of the 100 MHz constant clock so that every wave leaves the kernel even
-// if nobody ever raises the word.
+// Gate of a kernel on a host-visible word reaching seq.  Only block 0's leader
+// polls the host word (each poll crosses PCIe); it republishes the value in a
+// device word (`relay`) that the other blocks' leaders poll at L2 latency.  Block
+// 0 never waits on another block, so the gate cannot deadlock however many blocks
+// are resident.  Every wait is bounded by a tick count of the 100 MHz constant
+// clock, so every wave leaves the kernel even if nobody ever raises the word.
 __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsigned long long seq,
-                                          unsigned long long limit, unsigned long long* fp)
+                                          unsigned long long limit, unsigned long long* relay,
+                                          unsigned long long* fp)
 {
     if (threadIdx.x == 0) {
-        if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_IN, seq);
-        unsigned long long t0 = wall_clock64();
-        while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
-            __builtin_amdgcn_s_sleep(1);
-            if (wall_clock64() - t0 > limit) {
-                if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
-                break;
+        const unsigned long long t0 = wall_clock64();
+        if (blockIdx.x == 0 || !relay) {
+            if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_IN, seq);
+            while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
+                __builtin_amdgcn_s_sleep(1);
+                if (wall_clock64() - t0 > limit) {
+                    if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
+                    break;
+                }
+            }
+            if (relay) __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_OUT, seq);
+        } else {
+            while (__hip_atomic_load(relay, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < seq) {
+                __builtin_amdgcn_s_sleep(2);
+                if (wall_clock64() - t0 > limit + 100000000ull) break;
             }
         }
-        if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_OUT, seq);
     }
     __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");       // payload written before the flag is visible to all waves
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");       // the payload was written before the flag: no stale lines from here on
 }
 
 // ---------------------------------------------------------------- the step kernel
@@ -134,10 +175,10 @@ struct StepArgs {
     u32x4* bounce; unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long* tagp;
     // sum
     u32x4* out; const u32x4* b;
-    const unsigned long long* wait_flag; unsigned long long spin_limit;
+    const unsigned long long* wait_flag; unsigned long long* relay; unsigned long long spin_limit;
     unsigned long long* done; unsigned int* done_arrive;
     // common
-    const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp;
+    const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp; int sigmode;
 };
 
 template <int DT, int U, bool PACK, bool SUM>
@@ -145,26 +186,35 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 {
     const unsigned tid = threadIdx.x, nthr = blockDim.x;
     if (PACK && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
-    if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.fp);
+    if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
 
     const size_t nvec = g.nbytes >> 4;
     const size_t tile = (size_t)nthr * U;
     for (size_t base = (size_t)blockIdx.x * tile; base < nvec; base += (size_t)gridDim.x * tile) {
         u32x4 x[U], y[U];
+        if (base + tile <= nvec) {                       // whole tile: no per-vector bounds checks
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            size_t i = base + (size_t)u * nthr + tid;
-            if (i < nvec) {
+            for (int u = 0; u < U; u++) {
+                const size_t i = base + (size_t)u * nthr + tid;
                 x[u] = g.a[i];
                 if (SUM) y[u] = __builtin_nontemporal_load(g.b + i);
             }
-        }
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            size_t i = base + (size_t)u * nthr + tid;
-            if (i < nvec) {
+            for (int u = 0; u < U; u++) {
+                const size_t i = base + (size_t)u * nthr + tid;
                 if (PACK) g.bounce[i] = x[u];
                 if (SUM) g.out[i] = add_vec<DT>(x[u], y[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const size_t i = base + (size_t)u * nthr + tid;
+                if (i < nvec) {
+                    x[u] = g.a[i];
+                    if (SUM) y[u] = __builtin_nontemporal_load(g.b + i);
+                    if (PACK) g.bounce[i] = x[u];
+                    if (SUM) g.out[i] = add_vec<DT>(x[u], y[u]);
+                }
             }
         }
     }
@@ -186,10 +236,10 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
     }
     if (PACK) {
         if (g.tagp && blockIdx.x == 0 && tid == 0) *g.tagp = g.seq;
-        grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x);
+        grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
     }
     if (SUM && g.done) {
-        grid_complete(g.done, g.seq, g.done_arrive, gridDim.x);
+        grid_complete(g.done, g.seq, g.done_arrive, gridDim.x, 1);
     }
 }
 
@@ -206,19 +256,19 @@ __global__ __launch_bounds__(kThreads) void k_pack_narrow(PackArgs a)
     if (blockIdx.x == 0 && threadIdx.x < tail)
         ((unsigned char*)a.dst)[n * sizeof(W) + threadIdx.x] = ((const unsigned char*)a.src)[n * sizeof(W) + threadIdx.x];
     if (a.tagp && blockIdx.x == 0 && threadIdx.x == 0) *a.tagp = a.seq;
-    grid_complete(a.cflag, a.seq, a.arrive, gridDim.x);
+    grid_complete(a.cflag, a.seq, a.arrive, gridDim.x, a.sigmode);
 }
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void k_sum_narrow(SumArgs a)
 {
     typedef typename Elem<DT>::T T;
-    if (a.wait_flag) gate_wait(a.wait_flag, a.seq, a.spin_limit_ticks, a.fp);
+    if (a.wait_flag) gate_wait(a.wait_flag, a.seq, a.spin_limit_ticks, a.relay, a.fp);
     const size_t n = a.nbytes / sizeof(T);
     const T* x = (const T*)a.a; const T* y = (const T*)a.b; T* o = (T*)a.out;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
         o[i] = Elem<DT>::add(x[i], y[i]);
-    if (a.done) grid_complete(a.done, a.seq, a.done_arrive, gridDim.x);
+    if (a.done) grid_complete(a.done, a.seq, a.done_arrive, gridDim.x, 1);
 }
 
 // ---------------------------------------------------------------- diagnostics
@@ -226,7 +276,7 @@ __global__ __launch_bounds__(kThreads) void k_sum_narrow(SumArgs a)
 __global__ void k_waitflag(const unsigned long long* flag, unsigned long long seq, unsigned long long limit,
                            unsigned long long* fp)
 {
-    gate_wait(flag, seq, limit, fp);
+    gate_wait(flag, seq, limit, nullptr, fp);
 }
 
 // Re-reads the sequence tag the pack kernel appended to the payload, once with a
@@ -251,12 +301,12 @@ __global__ void k_fill_u32(unsigned int* p, unsigned int v, size_t n)
 
 // ---------------------------------------------------------------- launch geometry
 
-static int g_unroll = 4;        // vectors per lane per iteration for the large path
-static int g_grid_cap = kMaxGrid;
+static int g_unroll = 1;        // vectors per lane per iteration for the large path
+static int g_grid_cap = 1024;
 
 struct Geom { int grid, block, unroll; };
 
-static Geom geom_for(size_t nbytes)
+static Geom geom_for(size_t nbytes, bool writeback = false)
 {
     size_t nvec = nbytes >> 4;
     Geom g;
@@ -269,9 +319,12 @@ static Geom geom_for(size_t nbytes)
     }
     g.block = kThreads;
     g.unroll = (nvec >= (size_t)kThreads * 16) ? g_unroll : 1;
+    // an L2 write-back per block is dear and they run one after another: use one fat block per CU
+    const int cap = writeback ? 256 : g_grid_cap;
+    if (writeback) g.unroll = 8;
     size_t tile = (size_t)g.block * g.unroll;
     size_t tiles = (nvec + tile - 1) / tile;
-    g.grid = (int)(tiles < (size_t)g_grid_cap ? tiles : (size_t)g_grid_cap);
+    g.grid = (int)(tiles < (size_t)cap ? tiles : (size_t)cap);
     if (g.grid < 1) g.grid = 1;
     return g;
 }
@@ -282,73 +335,82 @@ int sum_grid(size_t nbytes, int) { return geom_for(nbytes).grid; }
 void set_tuning(int unroll, int grid_cap)
 {
     if (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) g_unroll = unroll;
-    if (grid_cap >= 1 && grid_cap <= 65535) g_grid_cap = grid_cap;
+    // the completion counters have one line per group of kGroup blocks: keep the grid within them
+    const int most = (int)(kGroup * (kCounterWords / kCtrLine - 1));
+    if (grid_cap >= 1) g_grid_cap = grid_cap < most ? grid_cap : most;
 }
 
 static inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
-template <int DT, bool PACK, bool SUM>
-static hipError_t launch_step_u(const StepArgs& s, const Geom& g, hipStream_t st)
+// One launch of a kernel that takes a single argument struct; with `t` the
+// dispatch's own start/end timestamps land in t->start / t->stop.
+template <typename A>
+static hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const Timing* t, const A& arg)
 {
-    switch (g.unroll) {
-        case 1: hipLaunchKernelGGL((k_step<DT, 1, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
-        case 2: hipLaunchKernelGGL((k_step<DT, 2, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
-        case 8: hipLaunchKernelGGL((k_step<DT, 8, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
-        default: hipLaunchKernelGGL((k_step<DT, 4, PACK, SUM>), dim3(g.grid), dim3(g.block), 0, st, s); break;
-    }
+    if (t && t->start && t->stop) hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, t->start, t->stop, 0, arg);
+    else hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, arg);
     return hipGetLastError();
 }
 
-template <bool PACK, bool SUM>
-static hipError_t launch_step(int dtype, const StepArgs& s, const Geom& g, hipStream_t st)
+template <int DT, bool PACK, bool SUM>
+static hipError_t launch_step_u(const StepArgs& s, const Geom& g, hipStream_t st, const Timing* t)
 {
-    if (!SUM) return launch_step_u<0, PACK, SUM>(s, g, st);      // the copy does not depend on the element type
+    switch (g.unroll) {
+        case 1: return launch1(k_step<DT, 1, PACK, SUM>, g.grid, g.block, st, t, s);
+        case 2: return launch1(k_step<DT, 2, PACK, SUM>, g.grid, g.block, st, t, s);
+        case 8: return launch1(k_step<DT, 8, PACK, SUM>, g.grid, g.block, st, t, s);
+        default: return launch1(k_step<DT, 4, PACK, SUM>, g.grid, g.block, st, t, s);
+    }
+}
+
+template <bool PACK, bool SUM>
+static hipError_t launch_step(int dtype, const StepArgs& s, const Geom& g, hipStream_t st, const Timing* t)
+{
+    if (!SUM) return launch_step_u<0, PACK, SUM>(s, g, st, t);      // the copy does not depend on the element type
     switch (dtype) {
-        case 0: return launch_step_u<0, PACK, SUM>(s, g, st);
-        case 1: return launch_step_u<1, PACK, SUM>(s, g, st);
-        case 2: return launch_step_u<2, PACK, SUM>(s, g, st);
+        case 0: return launch_step_u<0, PACK, SUM>(s, g, st, t);
+        case 1: return launch_step_u<1, PACK, SUM>(s, g, st, t);
+        case 2: return launch_step_u<2, PACK, SUM>(s, g, st, t);
     }
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_pack(const PackArgs& a, hipStream_t st)
+hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t)
 {
     if (!a.dst || !a.src || !a.cflag || !a.arrive || !al16(a.dst)) return hipErrorInvalidValue;
     if (al16(a.src)) {
         StepArgs s{};
         s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive; s.tagp = a.tagp;
-        s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
-        return launch_step<true, false>(0, s, geom_for(a.nbytes), st);
+        s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp; s.sigmode = a.sigmode;
+        return launch_step<true, false>(0, s, geom_for(a.nbytes, a.sigmode != 0), st, t);
     }
     size_t units = a.nbytes / 4 + 1;
-    int grid = (int)((units + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid;
-    if ((((uintptr_t)a.src) & 3) == 0) hipLaunchKernelGGL((k_pack_narrow<uint32_t>), dim3(grid), dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((k_pack_narrow<unsigned char>), dim3(grid), dim3(kThreads), 0, st, a);
-    return hipGetLastError();
+    int grid = (int)((units + kThreads - 1) / kThreads); if (grid > 1024) grid = 1024;
+    if ((((uintptr_t)a.src) & 3) == 0) return launch1(k_pack_narrow<uint32_t>, grid, kThreads, st, t, a);
+    return launch1(k_pack_narrow<unsigned char>, grid, kThreads, st, t, a);
 }
 
-hipError_t launch_sum(const SumArgs& a, hipStream_t st)
+hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
 {
     if (!a.out || !a.a || !a.b || a.dtype < 0 || a.dtype > 2) return hipErrorInvalidValue;
     if (a.done && !a.done_arrive) return hipErrorInvalidValue;
     if (al16(a.out) && al16(a.a) && al16(a.b)) {
         StepArgs s{};
-        s.out = (u32x4*)a.out; s.b = (const u32x4*)a.b; s.wait_flag = a.wait_flag; s.spin_limit = a.spin_limit_ticks;
+        s.out = (u32x4*)a.out; s.b = (const u32x4*)a.b; s.wait_flag = a.wait_flag; s.relay = a.relay; s.spin_limit = a.spin_limit_ticks;
         s.done = a.done; s.done_arrive = a.done_arrive;
         s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
-        return launch_step<false, true>(a.dtype, s, geom_for(a.nbytes), st);
+        return launch_step<false, true>(a.dtype, s, geom_for(a.nbytes), st, t);
     }
     size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
     int grid = (int)((n + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid; if (grid < 1) grid = 1;
     switch (a.dtype) {
-        case 0: hipLaunchKernelGGL((k_sum_narrow<0>), dim3(grid), dim3(kThreads), 0, st, a); break;
-        case 1: hipLaunchKernelGGL((k_sum_narrow<1>), dim3(grid), dim3(kThreads), 0, st, a); break;
-        default: hipLaunchKernelGGL((k_sum_narrow<2>), dim3(grid), dim3(kThreads), 0, st, a); break;
+        case 0: return launch1(k_sum_narrow<0>, grid, kThreads, st, t, a);
+        case 1: return launch1(k_sum_narrow<1>, grid, kThreads, st, t, a);
+        default: return launch1(k_sum_narrow<2>, grid, kThreads, st, t, a);
     }
-    return hipGetLastError();
 }
 
-hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st)
+hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
 {
     if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes)
         return hipErrorInvalidValue;
@@ -356,10 +418,10 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st)
     if (q.wait_flag) return hipErrorInvalidValue;     // waiting for the peer before sending to it would deadlock two real ranks
     StepArgs s{};
     s.bounce = (u32x4*)p.dst; s.cflag = p.cflag; s.pack_arrive = p.arrive; s.tagp = p.tagp;
-    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.spin_limit = q.spin_limit_ticks;
+    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
     s.done = q.done; s.done_arrive = q.done_arrive;
-    s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp;
-    return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes), st);
+    s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp; s.sigmode = p.sigmode;
+    return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes, p.sigmode != 0), st, t);
 }
 
 hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq, unsigned long long limit,

@@ -57,6 +57,8 @@ def _bind(so):
     l.tbv_emu_arrival_log.argtypes = [up, ctypes.POINTER(ci), sz]; l.tbv_emu_arrival_log.restype = sz
     l.tbv_emu_latency_probe.argtypes = [ci]; l.tbv_emu_latency_probe.restype = ci
     l.tbv_emu_latencies.argtypes = [dp, sz]; l.tbv_emu_latencies.restype = sz
+    l.tbv_emu_kernel_timing.argtypes = [ci]; l.tbv_emu_kernel_timing.restype = ci
+    l.tbv_emu_kernel_times.argtypes = [ci, dp, dp]; l.tbv_emu_kernel_times.restype = sz
     l.tbv_emu_tag_counts.argtypes = [up, up, up]; l.tbv_emu_tag_counts.restype = None
     l.tbv_ar_allreduce_chunked.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce_chunked.restype = ci
     l.tbv_emu_run_pack.argtypes = [vp, sz, ci, vp]; l.tbv_emu_run_pack.restype = ci
@@ -234,6 +236,17 @@ def arrival_log(max_n=1 << 16):
     r = (ctypes.c_int * max_n)()
     n = _lib.tbv_emu_arrival_log(s, r, max_n)
     return [(s[i], r[i]) for i in range(n)]
+
+
+def kernel_timing(on=True):
+    _lib.tbv_emu_kernel_timing(1 if on else 0)
+
+
+def kernel_times(which):
+    """(count, mean_us, min_us) of the recorded pack (0) or sum (1) launches; clears them."""
+    m, mn = ctypes.c_double(), ctypes.c_double()
+    n = _lib.tbv_emu_kernel_times(which, ctypes.byref(m), ctypes.byref(mn))
+    return n, m.value, mn.value
 
 
 def tag_counts():
