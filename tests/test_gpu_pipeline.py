@@ -1,0 +1,245 @@
+"""GPU tests of the protocol around the kernels: multi-rail chunked pipeline with a
+seeded arrival order, the async stress mix, the watchdog, and every mode switch."""
+import os
+import time
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import DT, bits_np, dev, first_diff, say, session
+from libtbvcoll_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_sum(orc, a, b):
+    return orc.sum_torch(a.cpu(), b.cpu())
+
+
+# ---------------------------------------------------------------- multi-rail chunked pipeline (64 MiB fp16)
+
+@pytest.mark.parametrize("railsum", [0, 1])
+def test_multirail_pipeline_seeded_arrival_order(orc, railsum):
+    """fp16 [8192x4096] = 64 MiB as 16 chunks of CAP = 4 MiB, 2 rails x NSLOT = 4; every
+    (chunk, rail) fragment arrives by side-stream copy + flag bump in a seeded random
+    order; the result must equal the single-shot sum bit for bit."""
+    nslot, cap, nchunks = 4, 4 << 20, 16
+    numel = nchunks * cap // 2
+    with session(rails=2, cap=cap, TBV_NSLOT=nslot, TBV_RAILSUM=railsum, TBV_WDOG=20) as tbv:
+        a = dev(synth.normal(41, numel), torch.float16)
+        p = dev(synth.normal(42, numel), torch.float16)
+        out = torch.empty_like(a)
+        script = synth.arrival_script(5, nchunks, 2, nslot - 1)
+        k, released, slots, rails = orc.ring_model([cap] * nchunks, script, nslot, 2, 98304, nslot - 1)
+        assert k == 2 * nchunks and sorted(x for x in released if x) == list(range(1, nchunks + 1))
+        tbv.arrival_script(script)
+        per = cap // 2
+        for c in range(nchunks):
+            tbv.stage_peer(p[c * per:(c + 1) * per])
+        say("pipeline railsum", railsum, "script", script)
+        assert tbv.all_reduce_chunked(a, out)
+        torch.cuda.synchronize()
+        assert not tbv.err()
+        # observed arrivals follow the script: k-th arrival came from rail script[k], in per-rail FIFO order
+        log = tbv.arrival_log()
+        assert [r for _, r in log] == script
+        for rail in (0, 1):
+            assert [s for s, r in log if r == rail] == list(range(1, nchunks + 1))
+        assert torch.equal(out, a + p)                               # single-shot sum, torch's kernel
+        assert first_diff(out, oracle_sum(orc, a, p)) is None        # and the CPU oracle, all 32 Mi elements
+        tbv.arrival_script([])
+
+
+def test_chunked_ragged_tail_and_mixed_rails(orc):
+    """A payload that is not a multiple of the cap, with a last chunk small enough to use one rail."""
+    cap = 256 << 10
+    with session(rails=2, cap=cap, TBV_NSLOT=3) as tbv:
+        for name in ("bf16", "f32"):
+            dt = DT[name]
+            esz = 2 if name != "f32" else 4
+            numel = (5 * cap + 6000) // esz
+            a = dev(synth.uniform(51, numel), dt); p = dev(synth.uniform(52, numel), dt)
+            out = torch.empty_like(a)
+            per = cap // esz
+            for c in range(6):
+                tbv.stage_peer(p[c * per:min((c + 1) * per, numel)])
+            assert tbv.all_reduce_chunked(a, out)
+            torch.cuda.synchronize()
+            assert first_diff(out, oracle_sum(orc, a, p)) is None
+        assert not tbv.err()
+
+
+# ---------------------------------------------------------------- async stress mix
+
+def test_async_stress_mix(orc):
+    """5,000 consecutive all-reduces, sizes uniform over {8 KB, 64 KB, 1 MB, 16 MB}, dtypes cycling
+    bf16/fp16/fp32, values U[-4,4] seeded per call, progress threads and the 10 s watchdog live, no
+    synchronisation between calls inside a window; every output is checked bit for bit against torch's
+    add on the regenerated inputs (as step4/test_stress.py:33-35) and every 50th against the CPU oracle."""
+    sizes = [8 << 10, 64 << 10, 1 << 20, 16 << 20]
+    dts = [torch.bfloat16, torch.float16, torch.float32]
+    ncalls, window = 5000, 100
+    pick = synth.bits32(2024, ncalls, 7)
+    with session(rails=2, cap=16 << 20, TBV_NSLOT=4, TBV_WDOG=10) as tbv:
+        bad, checked_oracle = [], 0
+        for w0 in range(0, ncalls, window):
+            keep = []
+            for it in range(w0, min(w0 + window, ncalls)):
+                nb = sizes[int(pick[it]) % 4]; dt = dts[it % 3]
+                numel = nb // (4 if dt == torch.float32 else 2)
+                x = synth.torch_hash_uniform(2 * it, numel).to(dt)
+                p = synth.torch_hash_uniform(2 * it + 1, numel).to(dt)
+                out = torch.empty_like(x)
+                tbv.stage_peer(p)
+                assert tbv.all_reduce(x, out)
+                keep.append((it, x, p, out))
+            torch.cuda.synchronize()
+            for it, x, p, out in keep:
+                if not torch.equal(out, x + p):
+                    bad.append(it)
+                if it % 50 == 0:
+                    assert first_diff(out, oracle_sum(orc, x, p)) is None, it
+                    checked_oracle += 1
+            if w0 % 1000 == 0:
+                say("stress mix", w0, "bad", len(bad))
+        assert not bad, (len(bad), bad[:5])
+        assert checked_oracle == ncalls // 50 and not tbv.err()
+        pre, xfer, post, enq, n = tbv.stats4()
+        assert n == ncalls and xfer > 0 and enq > 0                  # rail 0 saw every call
+        tbv.rails(); tbv.hist()
+
+
+# ---------------------------------------------------------------- watchdog (condition forced from the host)
+
+def test_watchdog_releases_gpu_and_error_is_sticky(orc):
+    """The peer never signals call 3: within TBV_WDOG seconds the progress thread must log, set the
+    error flag, still raise the GPU's flag (the stream drains), and every later call must fail."""
+    with session(rails=2, cap=1 << 20, TBV_WDOG=1) as tbv:
+        a = dev(synth.normal(1, 1 << 18), torch.bfloat16); p = dev(synth.normal(2, 1 << 18), torch.bfloat16)
+        out = torch.empty_like(a)
+        for _ in range(2):
+            tbv.stage_peer(p); assert tbv.all_reduce(a, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, a + p) and not tbv.err()
+        tbv.withhold(3, 1)                                           # rail 1 of call 3 is never signalled
+        tbv.stage_peer(p)
+        t0 = time.time()
+        assert tbv.all_reduce(a, out)                                # enqueue itself succeeds
+        torch.cuda.synchronize()                                     # returns: the flag was raised despite the error
+        dt = time.time() - t0
+        assert 0.8 < dt < 4.0, dt
+        assert tbv.err()
+        with pytest.raises(RuntimeError):
+            tbv.all_reduce(a, out)                                   # rc -1: unrecoverable (step4/libtbvcoll.cpp:419)
+        tbv.withhold(0, 0)
+
+
+# ---------------------------------------------------------------- every mode gives the same bits
+
+MODES = {
+    "kwait": {"TBV_KWAIT": 1},
+    "event": {"TBV_GPUSIG": 0},
+    "sync": {"TBV_ASYNC": 0},
+    "tag": {"TBV_TAG": 1},
+    "cached_bounce": {"TBV_UNCACHED": 0},
+    "uncached_both": {"TBV_UNCACHED": 3},
+    "railsum": {"TBV_RAILSUM": 1},
+    "fusewait": {"TBV_FUSEWAIT": 1 << 30},
+    "chunk": {"TBV_CHUNK": 65536},
+    "nslot2": {"TBV_NSLOT": 2},
+    "nslot32": {"TBV_NSLOT": 32},
+    "unroll4": {"TBV_UNROLL": 4, "TBV_GRIDCAP": 200},
+    "pin": {"TBV_CPU": 0},
+}
+
+
+@pytest.mark.parametrize("mode", sorted(MODES))
+def test_modes_bit_exact(orc, mode):
+    with session(rails=2, cap=4 << 20, **MODES[mode]) as tbv:
+        k = 0
+        for name in ("bf16", "f16", "f32"):
+            dt = DT[name]
+            for nb in (8192, 57344, 229376, 4 << 20):
+                numel = nb // (4 if name == "f32" else 2)
+                outs = []
+                for rep in range(6):                                  # back to back: slots get reused
+                    k += 1
+                    a = dev(synth.normal(1000 + k, numel), dt); p = dev(synth.normal(5000 + k, numel), dt)
+                    out = torch.empty_like(a)
+                    tbv.stage_peer(p)
+                    assert tbv.all_reduce(a, out)
+                    outs.append((a, p, out))
+                torch.cuda.synchronize()
+                for a, p, out in outs:
+                    assert torch.equal(out, a + p), (mode, name, nb)
+                assert first_diff(outs[-1][2], oracle_sum(orc, outs[-1][0], outs[-1][1])) is None
+        # mirror mode too (reads the send bounce back through the side stream)
+        a = dev(synth.normal(77, 300000), torch.float16)
+        out = torch.empty_like(a)
+        assert tbv.all_reduce(a, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, a + a)
+        assert not tbv.err()
+        if mode == "tag":
+            checks, bad_plain, bad_sys = tbv.tag_counts()
+            assert checks == k + 1 and bad_plain == 0 and bad_sys == 0
+
+
+def test_resident_peer_fused_and_unfused(orc):
+    """Early peer: payload already in the receive slots, flag up on entry; optional pack+sum fusion."""
+    n = 16 << 20
+    a = dev(synth.prefill_activations(100, n // 2), torch.bfloat16)
+    b = dev(synth.prefill_activations(101, n // 2), torch.bfloat16)
+    want = oracle_sum(orc, a, b)
+    for fuse in (0, 1):
+        with session(rails=2, cap=n, TBV_FUSE=fuse) as tbv:
+            tbv.peer_resident(b)
+            out = torch.empty_like(a)
+            for _ in range(9):
+                assert tbv.all_reduce(a, out)
+            torch.cuda.synchronize()
+            assert first_diff(out, want) is None
+            # the send bounce holds the local tensor in both variants
+            slot = tbv.seq() % 4
+            import ctypes
+            hip = ctypes.CDLL("libamdhip64.so.7")
+            hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+            img = torch.empty_like(a)
+            assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(slot), n, 3) == 0
+            assert torch.equal(img.view(torch.int16), a.view(torch.int16))
+            # a smaller call under the same resident payload, then a staged one overriding it
+            small = a[:4096].clone(); o2 = torch.empty_like(small)
+            assert tbv.all_reduce(small, o2)
+            p3 = dev(synth.normal(9, 4096), torch.bfloat16)
+            tbv.stage_peer(p3); o3 = torch.empty_like(small)
+            assert tbv.all_reduce(small, o3)
+            torch.cuda.synchronize()
+            assert torch.equal(o2, small + b[:4096]) and torch.equal(o3, small + p3)
+            tbv.peer_resident(None)
+            assert not tbv.err()
+
+
+def test_full_size_properties(orc):
+    """Size-independent properties at the 16 MiB bench shape: commutativity (swap local and peer),
+    x + 0 = x, x + (-x) = +0, and in-place equals out-of-place."""
+    n = 16 << 20
+    a = dev(synth.prefill_activations(100, n // 2), torch.bfloat16)
+    b = dev(synth.prefill_activations(101, n // 2), torch.bfloat16)
+    with session(rails=2, cap=n) as tbv:
+        o1 = torch.empty_like(a); o2 = torch.empty_like(a); o3 = torch.empty_like(a); o4 = torch.empty_like(a)
+        tbv.stage_peer(b); assert tbv.all_reduce(a, o1)
+        tbv.stage_peer(a); assert tbv.all_reduce(b, o2)
+        z = torch.zeros_like(a)
+        tbv.stage_peer(z); assert tbv.all_reduce(a, o3)
+        neg = -a
+        tbv.stage_peer(neg); assert tbv.all_reduce(a, o4)
+        c = a.clone()
+        tbv.stage_peer(b); assert tbv.all_reduce(c)
+        torch.cuda.synchronize()
+        assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+        assert torch.equal(o3, a)
+        assert int(o4.view(torch.int16).count_nonzero()) == 0         # +0 everywhere, never -0
+        assert torch.equal(c.view(torch.int16), o1.view(torch.int16))
+        assert first_diff(o1, oracle_sum(orc, a, b)) is None
+        assert not tbv.err()
