@@ -25,6 +25,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12                      # MI355X HBM3E, bytes/s
+# Bytes the sum kernel moves between L2 and memory per 16 MiB launch, from rocprofv3 counter runs of this
+# command (profiles/prefill16MiB_pmc_fetch_write.txt): FETCH_SIZE 16407.0 KiB x 1.9972 (what the counter
+# reads for a plain 16 MiB copy, 8203.5 KiB for 16384 KiB) + WRITE_SIZE 16384.0 KiB x 1.0.
+SUM_TRAFFIC_BYTES = int((16407.0 * (16384.0 / 8203.5) + 16384.0) * 1024)
 N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
 
@@ -138,6 +142,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
     ap.add_argument("--fuse", type=int, default=0, help="1: pack+sum in one kernel when the peer is resident (4N)")
+    ap.add_argument("--calibrate-copy", type=int, default=0,
+                    help="also run this many plain 16 MiB device copies (known 16 MiB read + 16 MiB written), "
+                         "so a counter run of this command holds a kernel of known traffic to scale by")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-decode", action="store_true")
     args = ap.parse_args()
@@ -153,6 +160,12 @@ def main():
     torch.cuda.set_device(0)
 
     pre = run_prefill(tbv, torch, synth, args.steps, args.warmup, bool(args.fuse))
+    if args.calibrate_copy:
+        src = torch.empty(N_PREFILL, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.calibrate_copy):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     n = N_PREFILL
     alg_step = (4 if args.fuse else 5) * n
     ms = pre["wall"] / args.steps * 1e3
@@ -168,7 +181,7 @@ def main():
                    "nslot": 4, "rails": 2, "accumulate": "f32, round to nearest even", "bit_exact_vs_torch_add": pre["ok"],
                    "host_enqueue_us_per_call": round(pre["enq_us"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None,
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None if args.fuse else SUM_TRAFFIC_BYTES,
                      "kernel": "pack+sum" if args.fuse else "sum", "algorithmic_bytes": dom_bytes,
                      "avg_launch_us": round(pre["sum_us"], 3), "min_launch_us": round(pre["sum_min_us"], 3),
                      "launches": pre["n_sum"]},

@@ -20,6 +20,38 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+// Cache hints of the four data streams (1 = non-temporal).  The received payload is
+// read exactly once; the others are left to the measured defaults below.
+#ifndef TBV_NT_A
+#define TBV_NT_A 0
+#endif
+#ifndef TBV_NT_B
+#define TBV_NT_B 1
+#endif
+#ifndef TBV_NT_OUT
+#define TBV_NT_OUT 0
+#endif
+#ifndef TBV_NT_BOUNCE
+#define TBV_NT_BOUNCE 1
+#endif
+
+__device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_a(const uint32_t __attribute__((ext_vector_type(4)))* p)
+{
+    return TBV_NT_A ? __builtin_nontemporal_load(p) : *p;
+}
+__device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_b(const uint32_t __attribute__((ext_vector_type(4)))* p)
+{
+    return TBV_NT_B ? __builtin_nontemporal_load(p) : *p;
+}
+__device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
+{
+    if (TBV_NT_OUT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+__device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
+{
+    if (TBV_NT_BOUNCE) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
 static constexpr int kThreads = 256;        // 4 wavefronts of 64
 static constexpr int kMaxSmallThreads = 1024;
 static constexpr int kMaxGrid = 256 * 8;     // 256 CUs, up to 8 resident blocks each
@@ -196,24 +228,24 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
-                x[u] = g.a[i];
-                if (SUM) y[u] = __builtin_nontemporal_load(g.b + i);
+                x[u] = ld_a(g.a + i);
+                if (SUM) y[u] = ld_b(g.b + i);
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
-                if (PACK) g.bounce[i] = x[u];
-                if (SUM) g.out[i] = add_vec<DT>(x[u], y[u]);
+                if (PACK) st_bounce(g.bounce + i, x[u]);
+                if (SUM) st_out(g.out + i, add_vec<DT>(x[u], y[u]));
             }
         } else {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
                 if (i < nvec) {
-                    x[u] = g.a[i];
-                    if (SUM) y[u] = __builtin_nontemporal_load(g.b + i);
-                    if (PACK) g.bounce[i] = x[u];
-                    if (SUM) g.out[i] = add_vec<DT>(x[u], y[u]);
+                    x[u] = ld_a(g.a + i);
+                    if (SUM) y[u] = ld_b(g.b + i);
+                    if (PACK) st_bounce(g.bounce + i, x[u]);
+                    if (SUM) st_out(g.out + i, add_vec<DT>(x[u], y[u]));
                 }
             }
         }
