@@ -88,6 +88,7 @@ def run_decode(tbv, torch, synth, iters, fusewait):
     os.environ["TBV_NSLOT"] = "4"
     os.environ["TBV_FUSE"] = "0"
     os.environ["TBV_FUSEWAIT"] = str(n) if fusewait else "0"
+    os.environ["TBV_DEFERSIG"] = "1" if fusewait else "0"
     tbv.shutdown()
     tbv.init(0, "rail0", "", cap_bytes=n)
     st = torch.cuda.Stream()
@@ -113,10 +114,12 @@ def run_decode(tbv, torch, synth, iters, fusewait):
     ok = all(bool(torch.equal(outs[k], locs[k] + peers[k])) for k in range(npeer)) and not tbv.err()
     tbv.latency_probe(False)
     tbv.shutdown()
-    os.environ["TBV_FUSEWAIT"] = "0"
+    os.environ.pop("TBV_FUSEWAIT", None)
+    os.environ.pop("TBV_DEFERSIG", None)
     return {"p50_us": round(pct(lat, 0.50), 2), "p99_us": round(pct(lat, 0.99), 2), "min_us": round(min(lat), 2),
             "samples": len(lat), "us_per_call_wall": round(wall / iters * 1e6, 2), "bit_exact": ok,
-            "gate": "in-kernel flag poll fused into the sum" if fusewait else "hipStreamWaitValue64",
+            "gate": "flag polled inside the sum kernel, pack signal deferred (library default for one-rail sizes)" if fusewait
+            else "hipStreamWaitValue64 (TBV_FUSEWAIT=0 TBV_DEFERSIG=0)",
             "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word"}
 
 

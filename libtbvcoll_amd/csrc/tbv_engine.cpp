@@ -115,6 +115,10 @@ struct Engine {
     std::vector<std::pair<uint64_t, int>> arrivals;
     std::atomic<int> probe{0};
     std::vector<double> latencies;
+    // a pack's completion word that its kernel did not raise: the next kernel on the same stream raises it
+    tbv::PreSignal pending;
+    hipStream_t pending_stream = nullptr;
+    int defer = 1;                            // allow deferring (TBV_DEFERSIG)
     // optional per-kernel timing with events on the caller's stream: [0]=pack, [1]=sum
     int ktime = 0;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> kev[2];
@@ -379,13 +383,15 @@ int configure(const char* devs, size_t cap)
     G.fuse = geti("TBV_FUSE", 0);
     // uncached bounce: waves only drain their stores; cached bounce: block leader writes the L2 back
     G.packsig = geti("TBV_PACKSIG", (G.uncached & 1) ? 0 : 1);
-    G.fusewait_max = getz("TBV_FUSEWAIT", 0);
+    // messages that travel on one rail poll their flag inside the sum kernel by default
+    G.fusewait_max = getz("TBV_FUSEWAIT", G.rail1max);
+    G.defer = geti("TBV_DEFERSIG", 1);
     G.stride = G.cap + (G.tag ? 4096 : 0);
     { size_t per_item = G.chunkb ? ((G.cap + G.chunkb - 1) / G.chunkb + 1) : 1;
       G.wr_hwm = (int)std::min<size_t>(96, (size_t)(G.nslot - 1) * per_item); if (G.wr_hwm < 1) G.wr_hwm = 1; }
     G.R = count_rails(devs);
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
-    tbv::set_tuning(geti("TBV_UNROLL", 0), geti("TBV_GRIDCAP", 0));
+    tbv::set_tuning(geti("TBV_UNROLL", 0), geti("TBV_GRIDCAP", 0), geti("TBV_BLOCK", 0));
     G.configured = 1;
     return 0;
 }
@@ -431,7 +437,7 @@ struct KTimer {
 };
 
 struct Call {
-    uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused;
+    uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused; bool deferred;
 };
 
 int wait_for_room(int R)
@@ -451,6 +457,29 @@ int wait_for_room(int R)
     return 0;
 }
 
+// The completion signal a kernel about to be launched on `st` has to deliver for its predecessor.
+tbv::PreSignal take_pending(hipStream_t st)
+{
+    tbv::PreSignal p;
+    if (G.pending.word) {
+        if (G.pending_stream == st) p = G.pending;
+        else (void)tbv::launch_mark(G.pending.word, 0, G.pending.seq, G.pending_stream);   // other stream: deliver it there
+        G.pending = tbv::PreSignal{};
+        G.pending_stream = nullptr;
+    }
+    return p;
+}
+
+// A deferred signal must not outlive the call that made it.
+int flush_pending()
+{
+    if (!G.pending.word) return 0;
+    hipError_t e = tbv::launch_mark(G.pending.word, 0, G.pending.seq, G.pending_stream);
+    G.pending = tbv::PreSignal{};
+    G.pending_stream = nullptr;
+    return e == hipSuccess ? 0 : -1;
+}
+
 // First half of a call: sequence number, slot, pack kernel, work items.
 // `sum_out`/`dtype` are only used when the pack can be fused with the sum.
 int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c)
@@ -462,6 +491,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
     c->seq = ++G.seq;
     c->slot = (int)(c->seq % (uint64_t)G.nslot);
     c->fused = false;
+    c->deferred = false;
 
     // whose payload plays the peer for this call
     const char* peer = nullptr;
@@ -492,6 +522,14 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         if (G.gpusig) {
             const bool can_fuse = G.fuse && c->resident && sum_out && !G.tag &&
                                   !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
+            // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
+            // When the next kernel on the stream is one of ours and will not wait behind a stream gate
+            // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
+            // completion word alone and that next kernel raises it first thing.
+            const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
+            c->deferred = G.defer && !can_fuse && !G.tag && G.kwait != 1 && G.can_wait_value &&
+                          !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
+            pa.pre = take_pending(st);
             if (can_fuse) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
@@ -500,8 +538,10 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (tbv::launch_pack_sum(pa, sa, st, kt.get()) != hipSuccess) FAIL("pack+sum kernel launch failed");
                 c->fused = true;
             } else {
+                if (c->deferred) pa.cflag = nullptr;
                 KTimer kt(0);
                 if (tbv::launch_pack(pa, st, kt.get()) != hipSuccess) FAIL("pack kernel launch failed");
+                if (c->deferred) { G.pending.word = cflag(c->slot); G.pending.seq = c->seq; G.pending_stream = st; }
             }
         } else {
             if (hipMemcpyAsync(slot_send(c->slot), ptr, nbytes, hipMemcpyDeviceToDevice, st) != hipSuccess) FAIL("copy into send slot failed");
@@ -550,11 +590,13 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         sa.wait_flag = gate; sa.relay = gate ? relay_word(c.slot) : nullptr; sa.spin_limit_ticks = spin_ticks;
         sa.fp = G.kwait ? footprints() : nullptr;
         if (probe && last) { sa.done = doneword(c.slot); sa.done_arrive = done_counters(c.slot); }
+        sa.pre = take_pending(st);
         KTimer kt(1);
         if (tbv::launch_sum(sa, st, kt.get()) != hipSuccess) FAIL("sum kernel launch failed");
         return 0;
     };
     auto gate_stream = [&](unsigned long long* flag) -> int {
+        if (flush_pending() != 0) FAIL("deferred signal launch failed");     // never park a pending signal behind a gate
         if (G.kwait == 1 || !G.can_wait_value) {
             if (tbv::launch_waitflag(flag, c.seq, spin_ticks, G.kwait ? footprints() : nullptr, st) != hipSuccess) FAIL("wait kernel launch failed");
         } else if (hipStreamWaitValue64(st, flag, c.seq, hipStreamWaitValueGte, 0xffffffffffffffffull) != hipSuccess)
@@ -581,7 +623,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         // The flag may already be up when the call is made (the peer was early): the payload is then in
         // place before the sum is even launched and the stream needs no gate at all.
         const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
-        const bool fusewait = G.async && !arrived && c.nbytes <= G.fusewait_max && !G.tag && G.kwait != 1;
+        const bool fusewait = G.async && !arrived && (c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1;
         if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
             if (tbv::launch_tagchk((const unsigned long long*)(rb + tag_offset(c.nbytes)), c.seq, dbgwords(), st) != hipSuccess)
@@ -685,6 +727,7 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     LOGF("  emulated peer on device %d; stream wait value %s, stream write value %s; uncached=%d tag=%d railsum=%d fuse=%d fusewait<=%zu",
          G.device, G.can_wait_value ? "yes" : "no (wait kernel)", G.can_write_value ? "yes" : "no (mark kernel)",
          G.uncached, G.tag, G.railsum, G.fuse, G.fusewait_max);
+    LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
     return 0;
 }
 
@@ -702,6 +745,7 @@ extern "C" int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype,
     Call c;
     if (enqueue_pack(ptr, outp, nbytes, dtype, st, &c) != 0) return -1;
     if (enqueue_wait_sum(ptr, outp, dtype, st, c) != 0) return -1;
+    if (flush_pending() != 0) FAIL("deferred signal launch failed");
     { std::lock_guard<std::mutex> lk(G.smx); G.t_enq += nowt() - te; }
     return 0;
 }
@@ -942,6 +986,7 @@ extern "C" void tbv_emu_shutdown(void)
         G.kev[w].clear(); G.kev_used[w] = 0;
     }
     G.ktime = 0;
+    G.pending = tbv::PreSignal{}; G.pending_stream = nullptr;
     G.staged.clear(); G.repeat = Staged{nullptr, 0}; G.resident_bytes = 0;
     G.script.clear(); G.turn.store(0); G.withhold_seq.store(0);
     { std::lock_guard<std::mutex> lk(G.logmx); G.arrivals.clear(); G.latencies.clear(); }
@@ -985,6 +1030,7 @@ extern "C" int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, in
             if (enqueue_pack((const char*)ptr + off, nullptr, len, dtype, st, &calls[i + depth]) != 0) return -1;
         }
     }
+    if (flush_pending() != 0) FAIL("deferred signal launch failed");
     { std::lock_guard<std::mutex> lk(G.smx); G.t_enq += nowt() - te; }
     return 0;
 }
@@ -995,6 +1041,7 @@ extern "C" int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* 
     tbv::PackArgs pa{};
     pa.dst = slot_send(slot); pa.src = src; pa.nbytes = nbytes;
     pa.cflag = word(W_MISC, 8 + slot % 16);          // a completion word nobody waits on
+    if (getenv("TBV_EXP_DEVWORD")) pa.cflag = relay_word(slot) + 4;
     pa.seq = 1; pa.arrive = pack_counters(slot); pa.sigmode = G.packsig;
     return tbv::launch_pack(pa, (hipStream_t)stream) == hipSuccess ? 0 : -1;
 }

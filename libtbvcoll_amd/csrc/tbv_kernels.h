@@ -11,16 +11,22 @@ namespace tbv {
 // started, sum done.
 enum Footprint { FP_WAIT_IN = 0, FP_WAIT_OUT = 1, FP_PACK = 2, FP_SUM_DONE = 3, FP_WAIT_TIMEOUT = 4 };
 
+// A completion word some earlier kernel on the same stream left unsignalled: the
+// next kernel stores `seq` to it as its first action (the earlier kernel is
+// complete by then, so its stores are globally visible).
+struct PreSignal { unsigned long long* word = nullptr; unsigned long long seq = 0; };
+
 struct PackArgs {
     void* dst;                  // send slot (16-byte aligned)
     const void* src;            // caller tensor
     size_t nbytes;
-    unsigned long long* cflag;  // host-visible completion word of the slot
+    unsigned long long* cflag;  // host-visible completion word of the slot; null: do not signal (deferred to the next kernel)
     unsigned long long seq;
     unsigned int* arrive;       // the slot's counter lines (kCounterWords words), all return to 0
     unsigned long long* tagp;   // where to store seq after the payload, or null
     unsigned long long* fp;     // footprints or null
     int sigmode;                // how block stores are made visible before the block is counted (see grid_complete)
+    PreSignal pre;
 };
 
 struct SumArgs {
@@ -38,6 +44,7 @@ struct SumArgs {
     unsigned long long* done;
     unsigned int* done_arrive;  // counter lines (kCounterWords words), all return to 0
     unsigned long long* fp;
+    PreSignal pre;
 };
 
 // Optional exact timing of one launch: the two events receive the start and end
@@ -50,8 +57,8 @@ static constexpr size_t kCounterWords = 16 * 128;
 // Launch geometry is exposed so the host can log and test it.
 int pack_grid(size_t nbytes);
 int sum_grid(size_t nbytes, int dtype);
-// Tuning knobs for experiments: vectors per lane per iteration (1,2,4,8) and the grid cap.
-void set_tuning(int unroll, int grid_cap);
+// Tuning knobs for experiments: vectors per lane per iteration (1,2,4,8), the grid cap, threads per block.
+void set_tuning(int unroll, int grid_cap, int block);
 
 hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullptr);

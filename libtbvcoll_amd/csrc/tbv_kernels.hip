@@ -137,6 +137,9 @@ static constexpr unsigned kCtrLine = 16;       // words per counter line (64 byt
 __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
                                               unsigned int* ctr, unsigned int nblk, int mode)
 {
+#ifdef TBV_EXP_NOSIG
+    return;
+#endif
     if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -211,12 +214,14 @@ struct StepArgs {
     unsigned long long* done; unsigned int* done_arrive;
     // common
     const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp; int sigmode;
+    unsigned long long* pre_word; unsigned long long pre_seq;
 };
 
 template <int DT, int U, bool PACK, bool SUM>
 __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 {
     const unsigned tid = threadIdx.x, nthr = blockDim.x;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);     // deferred signal of the kernel before
     if (PACK && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
     if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
 
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
     }
     if (PACK) {
         if (g.tagp && blockIdx.x == 0 && tid == 0) *g.tagp = g.seq;
-        grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
+        if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
     }
     if (SUM && g.done) {
         grid_complete(g.done, g.seq, g.done_arrive, gridDim.x, 1);
@@ -280,6 +285,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 template <typename W>
 __global__ __launch_bounds__(kThreads) void k_pack_narrow(PackArgs a)
 {
+    if (a.pre.word && blockIdx.x == 0 && threadIdx.x == 0) store_sys(a.pre.word, a.pre.seq);
     if (a.fp && blockIdx.x == 0 && threadIdx.x == 0) store_sys(a.fp + FP_PACK, a.seq);
     const size_t n = a.nbytes / sizeof(W);
     const W* s = (const W*)a.src; W* d = (W*)a.dst;
@@ -288,13 +294,14 @@ __global__ __launch_bounds__(kThreads) void k_pack_narrow(PackArgs a)
     if (blockIdx.x == 0 && threadIdx.x < tail)
         ((unsigned char*)a.dst)[n * sizeof(W) + threadIdx.x] = ((const unsigned char*)a.src)[n * sizeof(W) + threadIdx.x];
     if (a.tagp && blockIdx.x == 0 && threadIdx.x == 0) *a.tagp = a.seq;
-    grid_complete(a.cflag, a.seq, a.arrive, gridDim.x, a.sigmode);
+    if (a.cflag) grid_complete(a.cflag, a.seq, a.arrive, gridDim.x, a.sigmode);
 }
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void k_sum_narrow(SumArgs a)
 {
     typedef typename Elem<DT>::T T;
+    if (a.pre.word && blockIdx.x == 0 && threadIdx.x == 0) store_sys(a.pre.word, a.pre.seq);
     if (a.wait_flag) gate_wait(a.wait_flag, a.seq, a.spin_limit_ticks, a.relay, a.fp);
     const size_t n = a.nbytes / sizeof(T);
     const T* x = (const T*)a.a; const T* y = (const T*)a.b; T* o = (T*)a.out;
@@ -335,6 +342,7 @@ __global__ void k_fill_u32(unsigned int* p, unsigned int v, size_t n)
 
 static int g_unroll = 1;        // vectors per lane per iteration for the large path
 static int g_grid_cap = 1024;
+static int g_block = kThreads;
 
 struct Geom { int grid, block, unroll; };
 
@@ -349,7 +357,7 @@ static Geom geom_for(size_t nbytes, bool writeback = false)
         g.grid = 1; g.block = thr; g.unroll = 1;
         return g;
     }
-    g.block = kThreads;
+    g.block = g_block;
     g.unroll = (nvec >= (size_t)kThreads * 16) ? g_unroll : 1;
     // an L2 write-back per block is dear and they run one after another: use one fat block per CU
     const int cap = writeback ? 256 : g_grid_cap;
@@ -364,8 +372,9 @@ static Geom geom_for(size_t nbytes, bool writeback = false)
 int pack_grid(size_t nbytes) { return geom_for(nbytes).grid; }
 int sum_grid(size_t nbytes, int) { return geom_for(nbytes).grid; }
 
-void set_tuning(int unroll, int grid_cap)
+void set_tuning(int unroll, int grid_cap, int block)
 {
+    if (block == 256 || block == 512 || block == 1024) g_block = block;
     if (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) g_unroll = unroll;
     // the completion counters have one line per group of kGroup blocks: keep the grid within them
     const int most = (int)(kGroup * (kCounterWords / kCtrLine - 1));
@@ -409,11 +418,12 @@ static hipError_t launch_step(int dtype, const StepArgs& s, const Geom& g, hipSt
 
 hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t)
 {
-    if (!a.dst || !a.src || !a.cflag || !a.arrive || !al16(a.dst)) return hipErrorInvalidValue;
+    if (!a.dst || !a.src || (a.cflag && !a.arrive) || !al16(a.dst)) return hipErrorInvalidValue;
     if (al16(a.src)) {
         StepArgs s{};
         s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive; s.tagp = a.tagp;
         s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp; s.sigmode = a.sigmode;
+        s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
         return launch_step<true, false>(0, s, geom_for(a.nbytes, a.sigmode != 0), st, t);
     }
     size_t units = a.nbytes / 4 + 1;
@@ -431,6 +441,7 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
         s.out = (u32x4*)a.out; s.b = (const u32x4*)a.b; s.wait_flag = a.wait_flag; s.relay = a.relay; s.spin_limit = a.spin_limit_ticks;
         s.done = a.done; s.done_arrive = a.done_arrive;
         s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
+        s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
         return launch_step<false, true>(a.dtype, s, geom_for(a.nbytes), st, t);
     }
     size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
@@ -453,6 +464,7 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
     s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp; s.sigmode = p.sigmode;
+    s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
     return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes, p.sigmode != 0), st, t);
 }
 

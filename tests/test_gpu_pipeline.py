@@ -146,6 +146,10 @@ MODES = {
     "uncached_both": {"TBV_UNCACHED": 3},
     "railsum": {"TBV_RAILSUM": 1},
     "fusewait": {"TBV_FUSEWAIT": 1 << 30},
+    "stream_gate_only": {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0},
+    "no_defer": {"TBV_DEFERSIG": 0},
+    "fusewait_no_defer": {"TBV_FUSEWAIT": 1 << 30, "TBV_DEFERSIG": 0},
+    "block512": {"TBV_BLOCK": 512, "TBV_UNROLL": 2, "TBV_GRIDCAP": 256},
     "chunk": {"TBV_CHUNK": 65536},
     "nslot2": {"TBV_NSLOT": 2},
     "nslot32": {"TBV_NSLOT": 32},
