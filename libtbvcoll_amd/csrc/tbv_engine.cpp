@@ -32,6 +32,7 @@
 #include <vector>
 
 #include "../../include/tbvcoll.h"
+#include "tbv_dma.h"
 #include "tbv_kernels.h"
 
 namespace {
@@ -60,6 +61,8 @@ struct Item {
     size_t xbytes;            // bytes on the wire: payload, plus the tag when tagging
     const char* peer;         // staged peer payload, or null: mirror this rank's send slot
     bool resident;            // peer payload is already in the receive slot
+    bool host_wire;           // deposit with copy-engine transfers only (no GPU queue involved)
+    bool peer_is_host;        // the staged payload lives in pinned host memory
 };
 
 struct Rail {
@@ -70,12 +73,14 @@ struct Rail {
     bool started = false;
     hipStream_t wire = nullptr;               // side stream that plays the peer's writes
     size_t script_pos = 0;                    // next position to look at in the arrival script
+    char* stage = nullptr;                    // 64 bytes of pinned host memory for the host wire's tag word (made at init:
+                                              // a progress thread must not allocate while the GPU is gated)
     // per-rail transfer statistics (guarded by Engine::smx)
     double rl_post = 0, rl_arr = 0;
     uint64_t rl_n = 0;
 };
 
-struct Staged { const char* ptr; size_t nbytes; };
+struct Staged { const char* ptr; size_t nbytes; bool is_host; };
 
 struct Engine {
     // configuration
@@ -105,7 +110,8 @@ struct Engine {
     int nseen = 0;
     // emulated peer
     std::deque<Staged> staged;
-    Staged repeat{nullptr, 0};
+    Staged repeat{nullptr, 0, false};
+    char* stage_block = nullptr;
     size_t resident_bytes = 0;
     std::vector<int> script;
     std::atomic<size_t> turn{0};
@@ -119,6 +125,8 @@ struct Engine {
     tbv::PreSignal pending;
     hipStream_t pending_stream = nullptr;
     int defer = 1;                            // allow deferring (TBV_DEFERSIG)
+    int wire_mode = 0;                        // TBV_WIRE: 0 auto (probe each new caller stream), 1 stream, 2 host
+    std::vector<std::pair<void*, bool>> stream_wire;   // caller stream -> use the host wire
     // optional per-kernel timing with events on the caller's stream: [0]=pack, [1]=sum
     int ktime = 0;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> kev[2];
@@ -209,6 +217,32 @@ hipError_t stream_bump(hipStream_t st, unsigned long long* w, uint64_t v)
     return tbv::launch_mark(w, 0, v, st);
 }
 
+// Host wire deposit of one rail fragment (see wire_xfer): copy-engine transfers issued
+// and awaited by this thread.  No HIP call is made here: a HIP call from a progress
+// thread can block on a runtime lock held by the caller thread while that thread
+// waits for the very stream this transfer is meant to release.
+int host_deposit(Rail& x, const Item& it, size_t off, size_t len, double t0)
+{
+    if (!tbv::dma_ready()) { LOGF("rail%d: no copy-engine access for the host wire", x.idx); return -1; }
+    size_t n = len;
+    if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;        // staged payload has no tag
+    const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
+    const tbv::DmaSide side = (it.peer && it.peer_is_host) ? tbv::DMA_HOST : tbv::DMA_DEVICE;
+    auto left = [&]() { double r = G.wdog - (nowt() - t0); return r > 0.001 ? r : 0.001; };
+    int rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + off, tbv::DMA_DEVICE, src, side, n, left());
+    if (rc == 0 && it.peer && G.tag) {       // the peer's own tag travels at the end of its payload
+        const size_t to = tag_offset(it.nbytes);
+        if (to >= off && to < off + len) {
+            if (!x.stage) return -1;
+            memcpy(x.stage, &it.seq, 8);
+            rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + to, tbv::DMA_DEVICE, x.stage, tbv::DMA_HOST, 8, left());
+        }
+    }
+    if (rc == -2) LOGF("watchdog: rail%d host wire copy exceeded %.1fs seq=%llu", x.idx, G.wdog, (unsigned long long)it.seq);
+    else if (rc != 0) LOGF("rail%d host wire copy failed seq=%llu", x.idx, (unsigned long long)it.seq);
+    return rc == 0 ? 0 : -1;
+}
+
 // ---- the emulated transfer of one rail (replaces do_xfer_rail, step4/libtbvcoll.cpp:172-211) ----
 // Posts this rail's fragment of the peer payload into the receive slot and waits
 // for its arrival word.  Returns 0, or -1 on error / watchdog.
@@ -237,7 +271,14 @@ int wire_xfer(Rail& x, const Item& it)
     }
 
     const bool withheld = (G.withhold_seq.load() == it.seq && G.withhold_rail.load() == x.idx);
-    if (!it.resident) {
+    if (!it.resident && it.host_wire) {
+        // Host wire: the fragment goes device/host -> pinned staging -> receive slot with copy-engine
+        // transfers that the host waits for, and the host raises the arrival word itself.  Nothing is
+        // placed on a GPU compute queue, so this works even when the caller's gated stream and the side
+        // stream are multiplexed onto the same hardware queue.
+        if (host_deposit(x, it, off, len, t0) != 0) return -1;
+        if (!withheld) st_rel(aw, it.seq);
+    } else if (!it.resident) {
         const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
         size_t n = len;
         if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;   // staged payload has no tag
@@ -386,6 +427,8 @@ int configure(const char* devs, size_t cap)
     // messages that travel on one rail poll their flag inside the sum kernel by default
     G.fusewait_max = getz("TBV_FUSEWAIT", G.rail1max);
     G.defer = geti("TBV_DEFERSIG", 1);
+    { const char* e = getenv("TBV_WIRE");
+      G.wire_mode = (e && !strcmp(e, "stream")) ? 1 : (e && !strcmp(e, "host")) ? 2 : 0; }
     G.stride = G.cap + (G.tag ? 4096 : 0);
     { size_t per_item = G.chunkb ? ((G.cap + G.chunkb - 1) / G.chunkb + 1) : 1;
       G.wr_hwm = (int)std::min<size_t>(96, (size_t)(G.nslot - 1) * per_item); if (G.wr_hwm < 1) G.wr_hwm = 1; }
@@ -414,6 +457,8 @@ void free_slab(char* p, const SlabCache& cache)
 
 // ---- enqueue halves --------------------------------------------------------------------
 
+bool use_host_wire(hipStream_t st);
+
 // Event pair for one kernel launch when kernel timing is on (pool grows on demand).
 // The events are handed to the launch itself, so they carry that dispatch's own
 // start and end timestamps.
@@ -437,7 +482,7 @@ struct KTimer {
 };
 
 struct Call {
-    uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused; bool deferred;
+    uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused; bool deferred; bool host_wire;
 };
 
 int wait_for_room(int R)
@@ -492,19 +537,21 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
     c->slot = (int)(c->seq % (uint64_t)G.nslot);
     c->fused = false;
     c->deferred = false;
+    c->host_wire = G.async && use_host_wire(st);
 
     // whose payload plays the peer for this call
     const char* peer = nullptr;
+    bool peer_is_host = false;
     c->resident = false;
     if (!G.staged.empty()) {
         Staged s = G.staged.front(); G.staged.pop_front();
         if (s.nbytes < nbytes) FAIL("staged peer payload (%zu B) is shorter than the call (%zu B)", s.nbytes, nbytes);
-        peer = s.ptr;
+        peer = s.ptr; peer_is_host = s.is_host;
     } else if (G.resident_bytes >= nbytes && G.resident_bytes) {
         c->resident = true;
     } else if (G.repeat.ptr) {
         if (G.repeat.nbytes < nbytes) FAIL("repeat peer payload (%zu B) is shorter than the call (%zu B)", G.repeat.nbytes, nbytes);
-        peer = G.repeat.ptr;
+        peer = G.repeat.ptr; peer_is_host = G.repeat.is_host;
     }
 
     tbv::PackArgs pa{};
@@ -551,7 +598,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         for (int r = 0; r < c->R; r++) {
             Rail& x = G.rr[r];
             uint64_t h = x.q_head.load(std::memory_order_relaxed);
-            x.q[h % G.nslot] = Item{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident};
+            x.q[h % G.nslot] = Item{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, c->host_wire, peer_is_host};
             x.q_head.store(h + 1, std::memory_order_release);
         }
         wake(&G.cv_item);
@@ -566,7 +613,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             if (nowt() - tp > G.wdog) FAIL("watchdog: stream did not drain");
         }
         { std::lock_guard<std::mutex> lk(G.smx); G.t_pre += nowt() - tp; }
-        Item it{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident};
+        Item it{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, false, peer_is_host};
         for (int r = 0; r < c->R; r++) if (wire_xfer(G.rr[r], it) != 0) { G.err.store(1); FAIL("transfer failed"); }
         const double tdr = nowt();          // nothing to reap: the emulated sends complete with their arrival
         { std::lock_guard<std::mutex> lk(G.smx); G.t_drain += nowt() - tdr; }
@@ -635,6 +682,46 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
     if (G.kwait && tbv::launch_mark(footprints(), tbv::FP_SUM_DONE, c.seq, st) != hipSuccess) FAIL("footprint launch failed");
     { std::lock_guard<std::mutex> lk(G.smx); G.t_post += nowt() - tq; }
     return 0;
+}
+
+// Do this caller stream and a rail's side stream end up on the same hardware queue?  The runtime
+// multiplexes streams onto a few hardware queues; two streams on one queue run in submission order,
+// so a side-stream copy submitted after the caller's gate would sit behind the gate it is meant to
+// release.  Probe: a wait kernel bounded to 300 us goes on the caller's stream, the word it waits
+// for is raised from the side stream; on separate queues the wait ends at once, on a shared queue it
+// runs to its bound.  Every kernel involved exits by itself.
+bool shares_queue_with_wire(hipStream_t st)
+{
+    if (hipStreamSynchronize(st) != hipSuccess) { (void)hipGetLastError(); return true; }   // measure queues, not backlog
+    for (int r = 0; r < G.R; r++) {
+        unsigned long long* w = scratchword();
+        st_rel(w, 0);
+        if (tbv::launch_waitflag(w, 1, 30000ull, nullptr, st) != hipSuccess) return true;
+        const double t0 = nowt();
+        if (stream_bump(G.rr[r].wire, w, 1) != hipSuccess) { (void)hipStreamSynchronize(st); return true; }
+        while (hipStreamQuery(st) == hipErrorNotReady && nowt() - t0 < 0.05) { }
+        const double dt = nowt() - t0;
+        (void)hipStreamSynchronize(G.rr[r].wire);
+        (void)hipStreamSynchronize(st);
+        (void)hipGetLastError();
+        if (dt > 200e-6) {
+            LOGF("stream %p shares a hardware queue with rail%d's side stream (probe %.0f us): using the host wire for it",
+                 (void*)st, r, dt * 1e6);
+            return true;
+        }
+        LOGF("stream %p and rail%d's side stream run on separate hardware queues (probe %.0f us)", (void*)st, r, dt * 1e6);
+    }
+    return false;
+}
+
+bool use_host_wire(hipStream_t st)
+{
+    if (G.wire_mode == 2) return true;
+    if (G.wire_mode == 1) return false;
+    for (auto& p : G.stream_wire) if (p.first == (void*)st) return p.second;
+    const bool host = shares_queue_with_wire(st) && tbv::dma_ready();
+    G.stream_wire.emplace_back((void*)st, host);
+    return host;
 }
 
 void note_stream(void* stream, size_t nbytes)
@@ -706,6 +793,9 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
         if (hipStreamCreateWithFlags(&x.wire, hipStreamNonBlocking) != hipSuccess) FAIL("side stream creation failed");
     }
     for (int i = 0; i < MAXSLOT; i++) G.rails_done[i].store(0);
+    const bool dma = tbv::dma_init(G.recvbase, MAXRAIL);
+    if (hipHostMalloc((void**)&G.stage_block, 64 * MAXRAIL, hipHostMallocDefault) != hipSuccess) FAIL("pinned staging allocation failed");
+    for (int r = 0; r < MAXRAIL; r++) G.rr[r].stage = G.stage_block + 64 * r;
     // does a stream-ordered 64-bit write reach the host block? otherwise signal with a one-thread kernel
     G.can_write_value = 1;
     if (hipStreamWriteValue64(G.rr[0].wire, scratchword(), 0x5eedull, 0) != hipSuccess ||
@@ -727,6 +817,7 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     LOGF("  emulated peer on device %d; stream wait value %s, stream write value %s; uncached=%d tag=%d railsum=%d fuse=%d fusewait<=%zu",
          G.device, G.can_wait_value ? "yes" : "no (wait kernel)", G.can_write_value ? "yes" : "no (mark kernel)",
          G.uncached, G.tag, G.railsum, G.fuse, G.fusewait_max);
+    LOGF("  wire %s; copy-engine access for the host wire: %s", G.wire_mode == 1 ? "stream" : G.wire_mode == 2 ? "host" : "auto", dma ? "yes" : "no");
     LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
     return 0;
 }
@@ -832,6 +923,16 @@ extern "C" void tbv_ar_fini(void)
 
 // ========================================================================== C ABI, part 2
 
+namespace {
+// Asked once, on the caller's thread, when a payload is staged.
+bool pointer_is_host(const void* p)
+{
+    hipPointerAttribute_t at;
+    if (hipPointerGetAttributes(&at, p) != hipSuccess) { (void)hipGetLastError(); return true; }   // unknown to HIP: plain host memory
+    return at.type == hipMemoryTypeHost;
+}
+}  // namespace
+
 extern "C" int tbv_emu_configure(const char* devs, size_t cap)
 {
     if (G.inited) return 0;
@@ -862,14 +963,14 @@ extern "C" int tbv_emu_stage_peer(const void* src, size_t nbytes)
 {
     if (!G.inited || !src) return -1;
     if (G.staged.size() >= LOG_MAX) return -1;
-    G.staged.push_back(Staged{(const char*)src, nbytes});
+    G.staged.push_back(Staged{(const char*)src, nbytes, pointer_is_host(src)});
     return 0;
 }
 
 extern "C" int tbv_emu_stage_peer_repeat(const void* src, size_t nbytes)
 {
     if (!G.inited) return -1;
-    G.repeat = Staged{(const char*)src, src ? nbytes : 0};
+    G.repeat = Staged{(const char*)src, src ? nbytes : 0, src ? pointer_is_host(src) : false};
     return 0;
 }
 
@@ -976,6 +1077,9 @@ extern "C" void tbv_emu_shutdown(void)
     (void)hipDeviceSynchronize();
     tbv_ar_fini();
     for (int r = 0; r < G.R; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
+    for (int r = 0; r < MAXRAIL; r++) G.rr[r].stage = nullptr;
+    if (G.stage_block) { (void)hipHostFree(G.stage_block); G.stage_block = nullptr; }
+    G.stream_wire.clear();
     for (int i = 0; i < G.nslot; i++) if (G.ev[i]) { (void)hipEventDestroy(G.ev[i]); G.ev[i] = nullptr; }
     free_slab(G.sendbase, g_uc_send); G.sendbase = nullptr;
     free_slab(G.recvbase, g_uc_recv); G.recvbase = nullptr;
@@ -987,7 +1091,7 @@ extern "C" void tbv_emu_shutdown(void)
     }
     G.ktime = 0;
     G.pending = tbv::PreSignal{}; G.pending_stream = nullptr;
-    G.staged.clear(); G.repeat = Staged{nullptr, 0}; G.resident_bytes = 0;
+    G.staged.clear(); G.repeat = Staged{nullptr, 0, false}; G.resident_bytes = 0;
     G.script.clear(); G.turn.store(0); G.withhold_seq.store(0);
     { std::lock_guard<std::mutex> lk(G.logmx); G.arrivals.clear(); G.latencies.clear(); }
     G.probe.store(0);

@@ -150,6 +150,9 @@ MODES = {
     "no_defer": {"TBV_DEFERSIG": 0},
     "fusewait_no_defer": {"TBV_FUSEWAIT": 1 << 30, "TBV_DEFERSIG": 0},
     "block512": {"TBV_BLOCK": 512, "TBV_UNROLL": 2, "TBV_GRIDCAP": 256},
+    "host_wire": {"TBV_WIRE": "host"},
+    "host_wire_tag": {"TBV_WIRE": "host", "TBV_TAG": 1},
+    "stream_wire": {"TBV_WIRE": "stream"},
     "chunk": {"TBV_CHUNK": 65536},
     "nslot2": {"TBV_NSLOT": 2},
     "nslot32": {"TBV_NSLOT": 32},
@@ -247,3 +250,33 @@ def test_full_size_properties(orc):
         assert torch.equal(c.view(torch.int16), o1.view(torch.int16))
         assert first_diff(o1, oracle_sum(orc, a, b)) is None
         assert not tbv.err()
+
+
+def test_many_caller_streams_share_hardware_queues(orc):
+    """The runtime multiplexes streams onto a few hardware queues.  With more live streams than queues a
+    caller's gated stream and a rail's side stream can land on one queue, where a side-stream copy would
+    sit behind the gate it is meant to release.  The engine probes every new caller stream and moves such
+    streams to the host wire; every call must complete (no watchdog) and be exact."""
+    streams = [torch.cuda.Stream() for _ in range(10)]
+    with session(rails=2, cap=1 << 20, TBV_WDOG=5) as tbv:
+        k = 0
+        for rep in range(2):
+            for st in streams:
+                for nb in (8192, 1 << 20):
+                    k += 1
+                    a = dev(synth.normal(300 + k, nb // 2), torch.bfloat16); p = dev(synth.normal(900 + k, nb // 2), torch.bfloat16)
+                    out = torch.empty_like(a)
+                    torch.cuda.synchronize()
+                    with torch.cuda.stream(st):
+                        tbv.stage_peer(p)
+                        assert tbv.all_reduce(a, out)
+                    st.synchronize()
+                    assert not tbv.err(), (rep, k)
+                    assert torch.equal(out, a + p)
+        # pinned host memory as the peer's payload
+        hp = torch.from_numpy(synth.normal(5, 4096)).to(torch.bfloat16).pin_memory()
+        a = dev(synth.normal(6, 4096), torch.bfloat16); out = torch.empty_like(a)
+        tbv.stage_peer(hp)
+        assert tbv.all_reduce(a, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), oracle_sum(orc, a, hp))
