@@ -29,9 +29,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12                      # MI355X HBM3E, bytes/s
 # Bytes the sum kernel moves between L2 and memory per 16 MiB launch, from rocprofv3 counter runs of this
-# command (profiles/prefill16MiB_pmc_fetch_write.txt): FETCH_SIZE 16407.0 KiB x 1.9972 (what the counter
+# command (profiles/prefill16MiB_pmc_fetch_write.txt): FETCH_SIZE 16407.5 KiB x 1.9972 (what the counter
 # reads for a plain 16 MiB copy, 8203.5 KiB for 16384 KiB) + WRITE_SIZE 16384.0 KiB x 1.0.
-SUM_TRAFFIC_BYTES = int((16407.0 * (16384.0 / 8203.5) + 16384.0) * 1024)
+SUM_TRAFFIC_BYTES = int((16407.5 * (16384.0 / 8203.5) + 16384.0) * 1024)
 N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
 
