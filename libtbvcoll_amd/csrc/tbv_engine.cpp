@@ -88,6 +88,7 @@ struct Engine {
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     size_t cap = 0, stride = 0, rail1max = 96u * 1024u, chunkb = 0, fusewait_max = 0;
     double wdog = 10.0;
+    double tick_hz = 1e8;                     // rate of the constant clock the kernels bound their waits with
     int can_wait_value = 1, can_write_value = 1;
     // memory
     char* sendbase = nullptr;
@@ -272,9 +273,9 @@ int wire_xfer(Rail& x, const Item& it)
 
     const bool withheld = (G.withhold_seq.load() == it.seq && G.withhold_rail.load() == x.idx);
     if (!it.resident && it.host_wire) {
-        // Host wire: the fragment goes device/host -> pinned staging -> receive slot with copy-engine
-        // transfers that the host waits for, and the host raises the arrival word itself.  Nothing is
-        // placed on a GPU compute queue, so this works even when the caller's gated stream and the side
+        // Host wire: the fragment goes straight into the receive slot with a copy-engine transfer that
+        // this thread waits for, and this thread raises the arrival word itself.  Nothing is placed on
+        // one of our compute queues, so this works even when the caller's gated stream and the side
         // stream are multiplexed onto the same hardware queue.
         if (host_deposit(x, it, off, len, t0) != 0) return -1;
         if (!withheld) st_rel(aw, it.seq);
@@ -626,7 +627,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
 {
     if (c.fused) return 0;
     const char* rb = slot_recv(c.slot);
-    const unsigned long long spin_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * 1e8);
+    const unsigned long long spin_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);
     const bool probe = G.probe.load() != 0;
     const size_t esz = dtype == 0 ? 4 : 2;
 
@@ -696,7 +697,7 @@ bool shares_queue_with_wire(hipStream_t st)
     for (int r = 0; r < G.R; r++) {
         unsigned long long* w = scratchword();
         st_rel(w, 0);
-        if (tbv::launch_waitflag(w, 1, 30000ull, nullptr, st) != hipSuccess) return true;
+        if (tbv::launch_waitflag(w, 1, (unsigned long long)(300e-6 * G.tick_hz), nullptr, st) != hipSuccess) return true;
         const double t0 = nowt();
         if (stream_bump(G.rr[r].wire, w, 1) != hipSuccess) { (void)hipStreamSynchronize(st); return true; }
         while (hipStreamQuery(st) == hipErrorNotReady && nowt() - t0 < 0.05) { }
@@ -769,7 +770,10 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     if (hipGetDevice(&G.device) != hipSuccess) FAIL("no HIP device");
     { int v = 0;
       if (hipDeviceGetAttribute(&v, hipDeviceAttributeCanUseStreamWaitValue, G.device) != hipSuccess) v = 0;
-      G.can_wait_value = v; }
+      G.can_wait_value = v;
+      int khz = 0;
+      if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, G.device) == hipSuccess && khz > 0) G.tick_hz = khz * 1e3;
+      (void)hipGetLastError(); }
 
     const size_t span = G.stride * (size_t)G.nslot;
     if (!alloc_slab(&G.sendbase, span, (G.uncached & 1) != 0, g_uc_send)) FAIL("send bounce allocation failed (%zu B)", span);

@@ -39,7 +39,7 @@ struct SumArgs {
     const unsigned long long* wait_flag;
     unsigned long long* relay;  // device word: block 0 polls wait_flag and republishes it here for the other blocks
     unsigned long long seq;
-    unsigned long long spin_limit_ticks;   // bound of the in-kernel wait (100 MHz ticks)
+    unsigned long long spin_limit_ticks;   // bound of the in-kernel wait, in ticks of the device's constant wall clock
     // optional completion word (latency probe / footprint): last block stores seq
     unsigned long long* done;
     unsigned int* done_arrive;  // counter lines (kCounterWords words), all return to 0

@@ -172,8 +172,9 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
 // polls the host word (each poll crosses PCIe); it republishes the value in a
 // device word (`relay`) that the other blocks' leaders poll at L2 latency.  Block
 // 0 never waits on another block, so the gate cannot deadlock however many blocks
-// are resident.  Every wait is bounded by a tick count of the 100 MHz constant
-// clock, so every wave leaves the kernel even if nobody ever raises the word.
+// are resident.  Every wait is bounded by a tick count of the constant-rate wall
+// clock (100 MHz on gfx950; the host passes ticks computed from the device's
+// reported rate), so every wave leaves the kernel even if nobody raises the word.
 __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsigned long long seq,
                                           unsigned long long limit, unsigned long long* relay,
                                           unsigned long long* fp)
@@ -194,7 +195,7 @@ __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsign
         } else {
             while (__hip_atomic_load(relay, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < seq) {
                 __builtin_amdgcn_s_sleep(2);
-                if (wall_clock64() - t0 > limit + 100000000ull) break;
+                if (wall_clock64() - t0 > limit + limit / 8 + 1000000ull) break;
             }
         }
     }
