@@ -101,6 +101,7 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
     os.environ["TBV_FUSE"] = "0"
     os.environ["TBV_FUSEWAIT"] = str(n) if fusewait else "0"
     os.environ["TBV_DEFERSIG"] = "1" if fusewait else "0"
+    os.environ["TBV_ONEKERNEL"] = "1" if fusewait else "0"
     tbv.shutdown()
     tbv.init(0, "rail0", "", cap_bytes=n)
     npeer = 64
@@ -127,10 +128,11 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
     tbv.shutdown()
     os.environ.pop("TBV_FUSEWAIT", None)
     os.environ.pop("TBV_DEFERSIG", None)
+    os.environ.pop("TBV_ONEKERNEL", None)
     return {"p50_us": round(pct(lat, 0.50), 2), "p99_us": round(pct(lat, 0.99), 2), "min_us": round(min(lat), 2),
             "samples": len(lat), "us_per_call_wall": round(wall / iters * 1e6, 2), "bit_exact": ok,
-            "gate": "flag polled inside the sum kernel, pack signal deferred (library default for one-rail sizes)" if fusewait
-            else "hipStreamWaitValue64 (TBV_FUSEWAIT=0 TBV_DEFERSIG=0)",
+            "gate": "one kernel per call: pack, completion word, flag poll, sum (library default for one-rail sizes)" if fusewait
+            else "pack kernel, hipStreamWaitValue64, sum kernel (TBV_FUSEWAIT=0 TBV_DEFERSIG=0 TBV_ONEKERNEL=0)",
             "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word"}
 
 

@@ -126,6 +126,7 @@ struct Engine {
     tbv::PreSignal pending;
     hipStream_t pending_stream = nullptr;
     int defer = 1;                            // allow deferring (TBV_DEFERSIG)
+    int onekernel = 1;                        // small calls as one launch: pack, signal, flag poll, sum (TBV_ONEKERNEL)
     int wire_mode = 0;                        // TBV_WIRE: 0 auto (probe each new caller stream), 1 stream, 2 host
     std::vector<std::pair<void*, bool>> stream_wire;   // caller stream -> use the host wire
     // optional per-kernel timing with events on the caller's stream: [0]=pack, [1]=sum
@@ -428,6 +429,7 @@ int configure(const char* devs, size_t cap)
     // messages that travel on one rail poll their flag inside the sum kernel by default
     G.fusewait_max = getz("TBV_FUSEWAIT", G.rail1max);
     G.defer = geti("TBV_DEFERSIG", 1);
+    G.onekernel = geti("TBV_ONEKERNEL", 1);
     { const char* e = getenv("TBV_WIRE");
       G.wire_mode = (e && !strcmp(e, "stream")) ? 1 : (e && !strcmp(e, "host")) ? 2 : 0; }
     G.stride = G.cap + (G.tag ? 4096 : 0);
@@ -574,11 +576,28 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
             // completion word alone and that next kernel raises it first thing.
+            // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
+            // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
+            const bool one_kernel = G.onekernel && !can_fuse && sum_out && !G.tag && G.kwait != 1 && G.can_wait_value &&
+                                    !(G.railsum && c->R > 1) && nbytes <= G.fusewait_max &&
+                                    tbv::small_call_blocks(nbytes) <= tbv::kSmallCallMaxBlocks &&
+                                    !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
             const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
-            c->deferred = G.defer && !can_fuse && !G.tag && G.kwait != 1 && G.can_wait_value &&
+            c->deferred = G.defer && !can_fuse && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
             pa.pre = take_pending(st);
-            if (can_fuse) {
+            if (one_kernel) {
+                tbv::SumArgs sa{};
+                sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
+                if (!c->resident) {
+                    sa.wait_flag = gflag(c->slot); sa.relay = relay_word(c->slot);
+                    sa.spin_limit_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);
+                }
+                if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
+                KTimer kt(1);
+                if (tbv::launch_small_call(pa, sa, st, kt.get()) != hipSuccess) FAIL("one-kernel call launch failed");
+                c->fused = true;
+            } else if (can_fuse) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
@@ -822,6 +841,7 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
          G.device, G.can_wait_value ? "yes" : "no (wait kernel)", G.can_write_value ? "yes" : "no (mark kernel)",
          G.uncached, G.tag, G.railsum, G.fuse, G.fusewait_max);
     LOGF("  wire %s; copy-engine access for the host wire: %s", G.wire_mode == 1 ? "stream" : G.wire_mode == 2 ? "host" : "auto", dma ? "yes" : "no");
+    LOGF("  small calls (<= %zu B) in one kernel: %s", G.fusewait_max, G.onekernel ? "yes" : "no");
     LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
     return 0;
 }

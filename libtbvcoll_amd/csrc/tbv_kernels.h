@@ -65,6 +65,11 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullpt
 // One kernel that does pack (with completion signal) and sum: legal only when the
 // received payload is already in place.
 hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+// A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
+// blocks of 1024 lanes, one 16-byte vector per lane.
+static constexpr int kSmallCallMaxBlocks = 16;
+int small_call_blocks(size_t nbytes);
+hipError_t launch_small_call(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq,
                            unsigned long long spin_limit_ticks, unsigned long long* fp, hipStream_t st);
 hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, unsigned long long* dbg,

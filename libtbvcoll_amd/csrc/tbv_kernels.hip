@@ -285,6 +285,45 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
     }
 }
 
+// ---------------------------------------------------------------- the one-kernel small call
+//
+// A whole small call in one launch: pack this block's vectors into the bounce slot,
+// count the blocks and raise the pack's completion word, poll the flag, then sum with
+// the local vectors still in registers.  The signal precedes the wait inside the same
+// kernel, so two ranks running this against each other cannot wait for one another's
+// data before having sent their own.  One vector per lane; the host keeps the grid to
+// a handful of blocks so that all of them are resident together (a block that has
+// not started cannot be counted, and the counted total gates everyone's flag).
+template <int DT>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_small_call(StepArgs g)
+{
+    const unsigned tid = threadIdx.x;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    const size_t nvec = g.nbytes >> 4;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + tid;
+    const bool mine = i < nvec;
+    const unsigned tail = (unsigned)(g.nbytes & 15);
+    const size_t off = nvec << 4;
+    u32x4 x = {0, 0, 0, 0};
+    if (mine) { x = ld_a(g.a + i); st_bounce(g.bounce + i, x); }
+    if (tail && blockIdx.x == 0 && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
+    grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
+    if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    if (mine) st_out(g.out + i, add_vec<DT>(x, ld_b(g.b + i)));
+    if (tail && blockIdx.x == 0) {
+        typedef typename Elem<DT>::T T;
+        const unsigned ne = tail / sizeof(T);
+        if (tid < ne) {
+            const T* pa = (const T*)((const char*)g.a + off);
+            const T* pb = (const T*)((const char*)g.b + off);
+            T* po = (T*)((char*)g.out + off);
+            po[tid] = Elem<DT>::add(pa[tid], pb[tid]);
+        }
+    }
+    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, gridDim.x, 1);
+}
+
 // Fallback bodies for caller pointers that are not 16-byte aligned: element (sum)
 // or 4/1-byte (pack) grid-stride loops.  Same results, lower bandwidth.
 template <typename W>
@@ -471,6 +510,36 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
     s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp; s.sigmode = p.sigmode;
     s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
     return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes, p.sigmode != 0), st, t);
+}
+
+int small_call_blocks(size_t nbytes)
+{
+    const size_t nvec = nbytes >> 4;
+    return (int)((nvec + kMaxSmallThreads - 1) / kMaxSmallThreads) + (nvec == 0 ? 1 : 0);
+}
+
+hipError_t launch_small_call(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+{
+    if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes || !p.cflag ||
+        !p.arrive || q.dtype < 0 || q.dtype > 2)
+        return hipErrorInvalidValue;
+    if (q.done && !q.done_arrive) return hipErrorInvalidValue;
+    const int grid = small_call_blocks(p.nbytes);
+    if (grid > kSmallCallMaxBlocks) return hipErrorInvalidValue;
+    const size_t nvec = p.nbytes >> 4;
+    int block = grid > 1 ? kMaxSmallThreads : (int)((nvec + 63) / 64 * 64);
+    if (block < 64) block = 64;
+    StepArgs s{};
+    s.bounce = (u32x4*)p.dst; s.cflag = p.cflag; s.pack_arrive = p.arrive; s.tagp = nullptr;
+    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.done = q.done; s.done_arrive = q.done_arrive;
+    s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp; s.sigmode = p.sigmode;
+    s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
+    switch (q.dtype) {
+        case 0: return launch1(k_small_call<0>, grid, block, st, t, s);
+        case 1: return launch1(k_small_call<1>, grid, block, st, t, s);
+        default: return launch1(k_small_call<2>, grid, block, st, t, s);
+    }
 }
 
 hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq, unsigned long long limit,

@@ -146,8 +146,10 @@ MODES = {
     "uncached_both": {"TBV_UNCACHED": 3},
     "railsum": {"TBV_RAILSUM": 1},
     "fusewait": {"TBV_FUSEWAIT": 1 << 30},
-    "stream_gate_only": {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0},
+    "stream_gate_only": {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0, "TBV_ONEKERNEL": 0},
     "no_defer": {"TBV_DEFERSIG": 0},
+    "two_kernels": {"TBV_ONEKERNEL": 0},
+    "one_kernel_256k": {"TBV_FUSEWAIT": 262144},
     "fusewait_no_defer": {"TBV_FUSEWAIT": 1 << 30, "TBV_DEFERSIG": 0},
     "block512": {"TBV_BLOCK": 512, "TBV_UNROLL": 2, "TBV_GRIDCAP": 256},
     "host_wire": {"TBV_WIRE": "host"},
