@@ -1169,7 +1169,6 @@ extern "C" int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* 
     tbv::PackArgs pa{};
     pa.dst = slot_send(slot); pa.src = src; pa.nbytes = nbytes;
     pa.cflag = word(W_MISC, 8 + slot % 16);          // a completion word nobody waits on
-    if (getenv("TBV_EXP_DEVWORD")) pa.cflag = relay_word(slot) + 4;
     pa.seq = 1; pa.arrive = pack_counters(slot); pa.sigmode = G.packsig;
     return tbv::launch_pack(pa, (hipStream_t)stream) == hipSuccess ? 0 : -1;
 }

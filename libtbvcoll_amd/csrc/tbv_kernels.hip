@@ -141,9 +141,6 @@ static constexpr unsigned kCtrLine = 16;       // words per counter line (64 byt
 __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
                                               unsigned int* ctr, unsigned int nblk, int mode)
 {
-#ifdef TBV_EXP_NOSIG
-    return;
-#endif
     if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
