@@ -231,7 +231,12 @@ int host_deposit(Rail& x, const Item& it, size_t off, size_t len, double t0)
     const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
     const tbv::DmaSide side = (it.peer && it.peer_is_host) ? tbv::DMA_HOST : tbv::DMA_DEVICE;
     auto left = [&]() { double r = G.wdog - (nowt() - t0); return r > 0.001 ? r : 0.001; };
-    int rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + off, tbv::DMA_DEVICE, src, side, n, left());
+    // TBV_CHUNK: the fragment travels as several writes, the completion only after the last
+    // (step4/libtbvcoll.cpp:181-194)
+    const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
+    int rc = 0;
+    for (size_t o = 0; o < n && rc == 0; o += ck)
+        rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + off + o, tbv::DMA_DEVICE, src + o, side, std::min(ck, n - o), left());
     if (rc == 0 && it.peer && G.tag) {       // the peer's own tag travels at the end of its payload
         const size_t to = tag_offset(it.nbytes);
         if (to >= off && to < off + len) {
@@ -284,8 +289,12 @@ int wire_xfer(Rail& x, const Item& it)
         const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
         size_t n = len;
         if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;   // staged payload has no tag
-        if (n && hipMemcpyAsync(slot_recv(it.slot) + off, src, n, hipMemcpyDefault, x.wire) != hipSuccess) {
-            LOGF("rail%d peer deposit failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
+        // TBV_CHUNK: the fragment travels as several writes, the completion signal only after the last
+        // (step4/libtbvcoll.cpp:181-194)
+        const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
+        for (size_t o = 0; o < n; o += ck)
+            if (hipMemcpyAsync(slot_recv(it.slot) + off + o, src + o, std::min(ck, n - o), hipMemcpyDefault, x.wire) != hipSuccess) {
+                LOGF("rail%d peer deposit failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
         if (it.peer && G.tag) {              // the peer's own tag travels at the end of its payload
             size_t to = tag_offset(it.nbytes);
             if (to >= off && to < off + len &&

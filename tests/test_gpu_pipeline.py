@@ -154,6 +154,7 @@ MODES = {
     "block512": {"TBV_BLOCK": 512, "TBV_UNROLL": 2, "TBV_GRIDCAP": 256},
     "host_wire": {"TBV_WIRE": "host"},
     "host_wire_tag": {"TBV_WIRE": "host", "TBV_TAG": 1},
+    "host_wire_chunk": {"TBV_WIRE": "host", "TBV_CHUNK": 40000},
     "stream_wire": {"TBV_WIRE": "stream"},
     "chunk": {"TBV_CHUNK": 65536},
     "nslot2": {"TBV_NSLOT": 2},
