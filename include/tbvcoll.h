@@ -85,8 +85,10 @@ void tbv_ar_fini(void);
  */
 
 /* Queue the peer's payload for the next call that has none yet (FIFO, one entry per
- * call).  `src` is a device pointer or pinned host memory holding at least the
- * call's nbytes; it must stay valid until that call's result is complete.  Calls
+ * call).  `src` holds at least the call's nbytes.  A device pointer is read when
+ * the call's transfer runs and must stay valid until that call's result is
+ * complete; host memory is copied to the device right here (the emulated wire
+ * never reads host memory) and may be reused at once.  Calls
  * with no queued payload fall back to the repeat payload, then to mirror mode
  * (the peer sends back this rank's own bounce slot, so out = 2 * in). */
 int tbv_emu_stage_peer(const void* src, size_t nbytes);

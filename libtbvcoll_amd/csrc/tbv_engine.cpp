@@ -62,7 +62,6 @@ struct Item {
     const char* peer;         // staged peer payload, or null: mirror this rank's send slot
     bool resident;            // peer payload is already in the receive slot
     bool host_wire;           // deposit with copy-engine transfers only (no GPU queue involved)
-    bool peer_is_host;        // the staged payload lives in pinned host memory
 };
 
 struct Rail {
@@ -73,14 +72,12 @@ struct Rail {
     bool started = false;
     hipStream_t wire = nullptr;               // side stream that plays the peer's writes
     size_t script_pos = 0;                    // next position to look at in the arrival script
-    char* stage = nullptr;                    // 64 bytes of pinned host memory for the host wire's tag word (made at init:
-                                              // a progress thread must not allocate while the GPU is gated)
     // per-rail transfer statistics (guarded by Engine::smx)
     double rl_post = 0, rl_arr = 0;
     uint64_t rl_n = 0;
 };
 
-struct Staged { const char* ptr; size_t nbytes; bool is_host; };
+struct Staged { const char* ptr; size_t nbytes; bool owned; };
 
 struct Engine {
     // configuration
@@ -112,7 +109,8 @@ struct Engine {
     // emulated peer
     std::deque<Staged> staged;
     Staged repeat{nullptr, 0, false};
-    char* stage_block = nullptr;
+    // device copies of payloads that were staged from host memory: (buffer, last call that reads it; 0 = not yet assigned)
+    std::vector<std::pair<char*, uint64_t>> owned;
     size_t resident_bytes = 0;
     std::vector<int> script;
     std::atomic<size_t> turn{0};
@@ -219,31 +217,31 @@ hipError_t stream_bump(hipStream_t st, unsigned long long* w, uint64_t v)
     return tbv::launch_mark(w, 0, v, st);
 }
 
-// Host wire deposit of one rail fragment (see wire_xfer): copy-engine transfers issued
-// and awaited by this thread.  No HIP call is made here: a HIP call from a progress
-// thread can block on a runtime lock held by the caller thread while that thread
-// waits for the very stream this transfer is meant to release.
+// Host wire deposit of one rail fragment (see wire_xfer): device-to-device copy-engine
+// transfers issued and awaited by this thread.  Two rules keep it from ever waiting on the
+// stream it is meant to release.  No HIP call is made here: one can block on a runtime lock
+// held by the caller thread while that thread waits for the gated stream.  And nothing is
+// read from host memory: the runtime's host-to-device engine works in order, so a transfer
+// would queue behind a copy the caller has issued on the gated stream (payloads staged from
+// host memory are moved to the device when they are staged; the peer's tag, which equals this
+// rank's, is taken from this rank's send slot where the pack kernel wrote it).
 int host_deposit(Rail& x, const Item& it, size_t off, size_t len, double t0)
 {
     if (!tbv::dma_ready()) { LOGF("rail%d: no copy-engine access for the host wire", x.idx); return -1; }
     size_t n = len;
     if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;        // staged payload has no tag
     const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
-    const tbv::DmaSide side = (it.peer && it.peer_is_host) ? tbv::DMA_HOST : tbv::DMA_DEVICE;
     auto left = [&]() { double r = G.wdog - (nowt() - t0); return r > 0.001 ? r : 0.001; };
     // TBV_CHUNK: the fragment travels as several writes, the completion only after the last
     // (step4/libtbvcoll.cpp:181-194)
     const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
     int rc = 0;
     for (size_t o = 0; o < n && rc == 0; o += ck)
-        rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + off + o, tbv::DMA_DEVICE, src + o, side, std::min(ck, n - o), left());
+        rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + off + o, tbv::DMA_DEVICE, src + o, tbv::DMA_DEVICE, std::min(ck, n - o), left());
     if (rc == 0 && it.peer && G.tag) {       // the peer's own tag travels at the end of its payload
         const size_t to = tag_offset(it.nbytes);
-        if (to >= off && to < off + len) {
-            if (!x.stage) return -1;
-            memcpy(x.stage, &it.seq, 8);
-            rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + to, tbv::DMA_DEVICE, x.stage, tbv::DMA_HOST, 8, left());
-        }
+        if (to >= off && to < off + len)
+            rc = tbv::dma_copy(x.idx, slot_recv(it.slot) + to, tbv::DMA_DEVICE, slot_send(it.slot) + to, tbv::DMA_DEVICE, 8, left());
     }
     if (rc == -2) LOGF("watchdog: rail%d host wire copy exceeded %.1fs seq=%llu", x.idx, G.wdog, (unsigned long long)it.seq);
     else if (rc != 0) LOGF("rail%d host wire copy failed seq=%llu", x.idx, (unsigned long long)it.seq);
@@ -553,17 +551,17 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
 
     // whose payload plays the peer for this call
     const char* peer = nullptr;
-    bool peer_is_host = false;
     c->resident = false;
     if (!G.staged.empty()) {
         Staged s = G.staged.front(); G.staged.pop_front();
         if (s.nbytes < nbytes) FAIL("staged peer payload (%zu B) is shorter than the call (%zu B)", s.nbytes, nbytes);
-        peer = s.ptr; peer_is_host = s.is_host;
+        peer = s.ptr;
+        if (s.owned) for (auto& o : G.owned) if (o.first == s.ptr) o.second = c->seq;
     } else if (G.resident_bytes >= nbytes && G.resident_bytes) {
         c->resident = true;
     } else if (G.repeat.ptr) {
         if (G.repeat.nbytes < nbytes) FAIL("repeat peer payload (%zu B) is shorter than the call (%zu B)", G.repeat.nbytes, nbytes);
-        peer = G.repeat.ptr; peer_is_host = G.repeat.is_host;
+        peer = G.repeat.ptr;
     }
 
     tbv::PackArgs pa{};
@@ -627,7 +625,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         for (int r = 0; r < c->R; r++) {
             Rail& x = G.rr[r];
             uint64_t h = x.q_head.load(std::memory_order_relaxed);
-            x.q[h % G.nslot] = Item{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, c->host_wire, peer_is_host};
+            x.q[h % G.nslot] = Item{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, c->host_wire};
             x.q_head.store(h + 1, std::memory_order_release);
         }
         wake(&G.cv_item);
@@ -642,7 +640,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             if (nowt() - tp > G.wdog) FAIL("watchdog: stream did not drain");
         }
         { std::lock_guard<std::mutex> lk(G.smx); G.t_pre += nowt() - tp; }
-        Item it{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, false, peer_is_host};
+        Item it{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, false};
         for (int r = 0; r < c->R; r++) if (wire_xfer(G.rr[r], it) != 0) { G.err.store(1); FAIL("transfer failed"); }
         const double tdr = nowt();          // nothing to reap: the emulated sends complete with their arrival
         { std::lock_guard<std::mutex> lk(G.smx); G.t_drain += nowt() - tdr; }
@@ -826,8 +824,6 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     }
     for (int i = 0; i < MAXSLOT; i++) G.rails_done[i].store(0);
     const bool dma = tbv::dma_init(G.recvbase, MAXRAIL);
-    if (hipHostMalloc((void**)&G.stage_block, 64 * MAXRAIL, hipHostMallocDefault) != hipSuccess) FAIL("pinned staging allocation failed");
-    for (int r = 0; r < MAXRAIL; r++) G.rr[r].stage = G.stage_block + 64 * r;
     // does a stream-ordered 64-bit write reach the host block? otherwise signal with a one-thread kernel
     G.can_write_value = 1;
     if (hipStreamWriteValue64(G.rr[0].wire, scratchword(), 0x5eedull, 0) != hipSuccess ||
@@ -957,12 +953,46 @@ extern "C" void tbv_ar_fini(void)
 // ========================================================================== C ABI, part 2
 
 namespace {
-// Asked once, on the caller's thread, when a payload is staged.
 bool pointer_is_host(const void* p)
 {
     hipPointerAttribute_t at;
     if (hipPointerGetAttributes(&at, p) != hipSuccess) { (void)hipGetLastError(); return true; }   // unknown to HIP: plain host memory
     return at.type == hipMemoryTypeHost;
+}
+
+// Every rail has finished every call up to this sequence number.
+uint64_t calls_done()
+{
+    // each rail's tail counts the items it has completed; a call is done when all its rails are.  The
+    // cheap conservative answer: nothing is in flight when every queue is empty.
+    for (int r = 0; r < G.R; r++)
+        if (G.rr[r].q_head.load(std::memory_order_acquire) != G.rr[r].q_tail.load(std::memory_order_acquire)) return 0;
+    return G.seq;
+}
+
+// Device copies of host-staged payloads are released on the caller's thread once no call can read them.
+void reap_owned()
+{
+    if (G.owned.empty()) return;
+    const uint64_t done = calls_done();
+    if (!done) return;
+    size_t k = 0;
+    for (auto& o : G.owned) {
+        if (o.second && o.second <= done) (void)hipFree(o.first);
+        else G.owned[k++] = o;
+    }
+    G.owned.resize(k);
+}
+
+// A payload in host memory is moved to the device when it is staged (see host_deposit for why the
+// wire never reads host memory).  Returns the device pointer, or null on failure.
+const char* to_device(const void* src, size_t nbytes)
+{
+    char* d = nullptr;
+    if (hipMalloc((void**)&d, nbytes ? nbytes : 1) != hipSuccess) return nullptr;
+    if (nbytes && hipMemcpy(d, src, nbytes, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(d); return nullptr; }
+    G.owned.emplace_back(d, 0);
+    return d;
 }
 }  // namespace
 
@@ -996,14 +1026,19 @@ extern "C" int tbv_emu_stage_peer(const void* src, size_t nbytes)
 {
     if (!G.inited || !src) return -1;
     if (G.staged.size() >= LOG_MAX) return -1;
-    G.staged.push_back(Staged{(const char*)src, nbytes, pointer_is_host(src)});
+    reap_owned();
+    const bool host = pointer_is_host(src);
+    const char* p = host ? to_device(src, nbytes) : (const char*)src;
+    if (!p) return -1;
+    G.staged.push_back(Staged{p, nbytes, host});
     return 0;
 }
 
 extern "C" int tbv_emu_stage_peer_repeat(const void* src, size_t nbytes)
 {
     if (!G.inited) return -1;
-    G.repeat = Staged{(const char*)src, src ? nbytes : 0, src ? pointer_is_host(src) : false};
+    if (src && pointer_is_host(src)) { src = to_device(src, nbytes); if (!src) return -1; G.owned.back().second = ~0ull; }   // kept until shutdown
+    G.repeat = Staged{(const char*)src, src ? nbytes : 0, false};
     return 0;
 }
 
@@ -1110,8 +1145,8 @@ extern "C" void tbv_emu_shutdown(void)
     (void)hipDeviceSynchronize();
     tbv_ar_fini();
     for (int r = 0; r < G.R; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
-    for (int r = 0; r < MAXRAIL; r++) G.rr[r].stage = nullptr;
-    if (G.stage_block) { (void)hipHostFree(G.stage_block); G.stage_block = nullptr; }
+    for (auto& o : G.owned) (void)hipFree(o.first);
+    G.owned.clear();
     G.stream_wire.clear();
     for (int i = 0; i < G.nslot; i++) if (G.ev[i]) { (void)hipEventDestroy(G.ev[i]); G.ev[i] = nullptr; }
     free_slab(G.sendbase, g_uc_send); G.sendbase = nullptr;
