@@ -204,6 +204,8 @@ def main():
                                "receive slots; values N(0,0.02^2) with 0.1% outliers at +-8",
                    "step": "pack+sum fused (4N)" if args.fuse else "pack 2N + flag wait + sum 3N = 5N",
                    "nslot": 4, "rails": 2, "accumulate": "f32, round to nearest even", "bit_exact_vs_torch_add": pre["ok"],
+                   "residency": "everything a step touches (local 16 + bounce ring 64 + receive ring 64 + out 16 MiB) fits the "
+                                "256 MB Infinity Cache; cache_cold in this line is the same step with the buffers rotated beyond it",
                    "host_enqueue_us_per_call": round(pre["enq_us"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None if args.fuse else SUM_TRAFFIC_BYTES,
