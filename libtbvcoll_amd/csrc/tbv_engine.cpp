@@ -602,14 +602,18 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 }
                 if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
                 KTimer kt(1);
+                const double tq = nowt();
                 if (tbv::launch_small_call(pa, sa, st, kt.get()) != hipSuccess) FAIL("one-kernel call launch failed");
+                { std::lock_guard<std::mutex> lk(G.smx); G.t_post += nowt() - tq; }      // the launch that carries the sum
                 c->fused = true;
             } else if (can_fuse) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
                 KTimer kt(1);
+                const double tq = nowt();
                 if (tbv::launch_pack_sum(pa, sa, st, kt.get()) != hipSuccess) FAIL("pack+sum kernel launch failed");
+                { std::lock_guard<std::mutex> lk(G.smx); G.t_post += nowt() - tq; }
                 c->fused = true;
             } else {
                 if (c->deferred) pa.cflag = nullptr;

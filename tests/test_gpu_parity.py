@@ -186,3 +186,57 @@ def test_mirror_mode_and_send_slot_image(orc):
                 assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(slot), nb, 3) == 0
                 want = orc.pack(a.cpu().contiguous().view(torch.uint8).numpy())
                 assert np.array_equal(img.cpu().numpy(), want)
+
+
+# ---------------------------------------------------------------- counterpart of step4/test_tbvcoll.py
+
+def test_latency_and_phase_breakdown(orc, capfd):
+    """In place on constant rank+1 tensors (1.0 here, 2.0 from the peer -> 3.0), 30 warm-up calls,
+    then timed calls per size; the phase averages and the stderr dumps behave as the reference's:
+    per-call averages, reset on read, histogram by log2 size, per-rail lines."""
+    import re
+    import time
+    sizes = [4096, 57344, 229376, 1048576]
+    iters = 300
+    with session(rails=2, cap=max(sizes)) as tbv:
+        for dt in (torch.float32, torch.bfloat16):
+            for nb in sizes:
+                numel = nb // torch.tensor([], dtype=dt).element_size()
+                peer = torch.full((numel,), 2.0, dtype=dt, device="cuda")
+                tbv.stage_peer_repeat(peer)
+                t = torch.full((numel,), 1.0, dtype=dt, device="cuda")
+                for _ in range(30):
+                    assert tbv.all_reduce(t)
+                    t.fill_(1.0)
+                torch.cuda.synchronize()
+                tbv.stats4()
+                t0 = time.perf_counter()
+                for _ in range(iters):
+                    tbv.all_reduce(t)
+                    t.fill_(1.0)
+                torch.cuda.synchronize()
+                tot = (time.perf_counter() - t0) / iters
+                pre, xfer, post, enq, n = tbv.stats4()
+                assert n == iters and pre == 0.0 and 0 < xfer < 5e4 and 0 < post < enq < 1e4
+                assert tbv.stats4() == (0.0, 0.0, 0.0, 0.0, 0)          # reading resets
+                c = torch.full((numel,), 1.0, dtype=dt, device="cuda")
+                assert tbv.all_reduce(c)
+                torch.cuda.synchronize()
+                assert torch.equal(c, torch.full_like(c, 3.0))           # exactly 3, not just close to it
+                say("phases", dt, nb, f"total {tot * 1e6:.1f} us enq {enq:.1f} xfer {xfer:.1f} post {post:.1f} "
+                    f"algbw {nb * 8 / tot / 1e9:.2f} Gb/s")
+        capfd.readouterr()
+        tbv.rails()
+        tbv.hist()
+        err = capfd.readouterr().err
+        calls_per_size = 2 * (30 + iters + 1)
+        # sizes 4096 and 57344 travel on one rail, the larger two on both
+        assert re.search(r"rail0: post +[\d.]+ +arrival +[\d.]+ +\(%d calls\)" % (4 * calls_per_size), err), err
+        assert re.search(r"rail1: post +[\d.]+ +arrival +[\d.]+ +\(%d calls\)" % (2 * calls_per_size), err), err
+        for nb, rails in ((4096, 1.0), (57344, 1.0), (229376, 2.0), (1048576, 2.0)):
+            bucket = 1 << (nb.bit_length() - 1)
+            m = re.search(r" +%d B~ : +(\d+) calls  mean +[\d.]+ us  mean rails ([\d.]+)" % bucket, err)
+            assert m and int(m.group(1)) == calls_per_size and float(m.group(2)) == rails, (nb, err)
+        tbv.hist()
+        assert " B~ :" not in capfd.readouterr().err                      # the dump reset the histogram
+        tbv.stage_peer_repeat(None)
