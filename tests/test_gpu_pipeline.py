@@ -283,3 +283,66 @@ def test_many_caller_streams_share_hardware_queues(orc):
         assert tbv.all_reduce(a, out)
         torch.cuda.synchronize()
         assert torch.equal(out.cpu(), oracle_sum(orc, a, hp))
+
+
+@pytest.mark.parametrize("seed,env", [(1, {}), (2, {"TBV_RAILSUM": 1}), (3, {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0, "TBV_ONEKERNEL": 0}),
+                                      (4, {"TBV_WIRE": "host"}), (5, {"TBV_FUSEWAIT": 262144, "TBV_NSLOT": 2})])
+def test_seeded_mix_of_everything(orc, seed, env):
+    """1500 calls drawn from a seeded stream: sizes from 2 bytes to the cap including odd element counts,
+    three dtypes, in place or not, aligned or offset pointers, peer staged / mirrored, two caller streams
+    used alternately (synchronised when switching, as a caller must), occasional chunked calls over the
+    cap.  Every result is compared with torch's add of the same operands; every 25th with the oracle."""
+    cap = 1 << 20
+    r = synth.bits32(7000 + seed, 1500 * 8, 7).reshape(1500, 8)
+    dts = [torch.bfloat16, torch.float16, torch.float32]
+    streams = [torch.cuda.current_stream(), torch.cuda.Stream()]
+    with session(rails=2, cap=cap, **env) as tbv:
+        cur = 0
+        pend = []
+        for it in range(1500):
+            q = [int(v) for v in r[it]]
+            dt = dts[q[0] % 3]
+            esz = 4 if dt == torch.float32 else 2
+            kind = q[1] % 10
+            if kind < 3:
+                numel = 1 + q[2] % 300
+            elif kind < 8:
+                numel = 1 + q[2] % (cap // esz)
+            elif kind == 8:
+                numel = cap // esz
+            else:
+                numel = cap // esz + 1 + q[2] % (3 * cap // esz)      # over the cap: chunked entry point
+            off = (q[3] % 4) if q[3] % 5 == 0 else 0
+            inplace = q[4] % 4 == 0
+            mirror = q[5] % 7 == 0
+            if q[6] % 40 == 0:                                         # switch streams the way a caller must
+                torch.cuda.synchronize()
+                cur ^= 1
+            chunked = numel * esz > cap
+            with torch.cuda.stream(streams[cur]):
+                base = synth.torch_hash_uniform(10 * it + seed, numel + 4).to(dt)
+                a = base[off:off + numel]
+                p = None if mirror else synth.torch_hash_uniform(10 * it + 5 + seed, numel).to(dt)
+                want = a + (a if mirror else p)
+                keep_a = a.clone() if it % 25 == 0 else None       # operands for the oracle (a is overwritten in place)
+                out = a if inplace else torch.empty(numel + 4, dtype=dt, device="cuda")[off:off + numel]
+                if p is not None:
+                    if chunked:
+                        per = cap // esz
+                        for c0 in range(0, numel, per):
+                            tbv.stage_peer(p[c0:min(c0 + per, numel)])
+                    else:
+                        tbv.stage_peer(p)
+                if chunked:
+                    assert tbv.all_reduce_chunked(a, None if inplace else out)
+                else:
+                    assert tbv.all_reduce(a, None if inplace else out)
+                pend.append((it, out, want, base, p, keep_a))
+            if len(pend) >= 64 or it == 1499:
+                torch.cuda.synchronize()
+                for k, o, w, _, pp, ka in pend:
+                    assert torch.equal(o, w), (seed, k, o.numel(), o.dtype)
+                    if ka is not None:
+                        assert first_diff(o, oracle_sum(orc, ka, ka if pp is None else pp)) is None
+                pend = []
+        assert not tbv.err()
