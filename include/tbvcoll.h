@@ -109,7 +109,9 @@ int tbv_emu_peer_resident(const void* src, size_t nbytes);
 int tbv_emu_arrival_script(const int* rails, size_t n);
 
 /* Fault injection from the host: the peer never signals rail `rail` of call `seq`
- * (seq counts calls from 1).  The watchdog must then trip.  seq == 0 clears. */
+ * (seq counts calls from 1); with rail == -1 it is the pack kernel of call `seq`
+ * that never raises its completion word.  The watchdog must then trip.
+ * seq == 0 clears. */
 int tbv_emu_withhold(unsigned long long seq, int rail);
 
 /* Sequence number of the last call issued (0 before the first). */
@@ -148,6 +150,11 @@ size_t tbv_emu_latencies(double* us, size_t max);
  * launches and their mean and minimum duration in microseconds, then forgets them. */
 int tbv_emu_kernel_timing(int on);
 size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_us);
+
+/* GPU footprints (kept with TBV_KWAIT=1, as the reference's, step4/libtbvcoll.cpp:98):
+ * sequence numbers of the last [wait entered, wait passed, pack started, sum done,
+ * wait that ran into its bound]. */
+void tbv_emu_footprints(unsigned long long out[5]);
 
 /* Stale-data detector counters (TBV_TAG=1): checks, plain-load mismatches,
  * system-scope-load mismatches. */

@@ -593,7 +593,13 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             c->deferred = G.defer && !can_fuse && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
             pa.pre = take_pending(st);
-            if (one_kernel) {
+            // fault injection from the host: this call's pack never raises its completion word
+            const bool mute_pack = G.withhold_seq.load() == c->seq && G.withhold_rail.load() < 0;
+            if (mute_pack) {
+                pa.cflag = nullptr;
+                c->deferred = false;
+                if (tbv::launch_pack(pa, st) != hipSuccess) FAIL("pack kernel launch failed");
+            } else if (one_kernel) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 if (!c->resident) {
@@ -1131,6 +1137,11 @@ extern "C" size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_u
     if (mean_us) *mean_us = n ? sum / (double)n : 0.0;
     if (min_us) *min_us = n ? mn : 0.0;
     return n;
+}
+
+extern "C" void tbv_emu_footprints(unsigned long long out[5])
+{
+    for (int i = 0; i < 5; i++) out[i] = G.inited ? footprints()[i] : 0;
 }
 
 extern "C" void tbv_emu_tag_counts(unsigned long long* checks, unsigned long long* bad_plain, unsigned long long* bad_system)

@@ -59,6 +59,7 @@ def _bind(so):
     l.tbv_emu_latencies.argtypes = [dp, sz]; l.tbv_emu_latencies.restype = sz
     l.tbv_emu_kernel_timing.argtypes = [ci]; l.tbv_emu_kernel_timing.restype = ci
     l.tbv_emu_kernel_times.argtypes = [ci, dp, dp]; l.tbv_emu_kernel_times.restype = sz
+    l.tbv_emu_footprints.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]; l.tbv_emu_footprints.restype = None
     l.tbv_emu_tag_counts.argtypes = [up, up, up]; l.tbv_emu_tag_counts.restype = None
     l.tbv_ar_allreduce_chunked.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce_chunked.restype = ci
     l.tbv_emu_run_pack.argtypes = [vp, sz, ci, vp]; l.tbv_emu_run_pack.restype = ci
@@ -247,6 +248,13 @@ def kernel_times(which):
     m, mn = ctypes.c_double(), ctypes.c_double()
     n = _lib.tbv_emu_kernel_times(which, ctypes.byref(m), ctypes.byref(mn))
     return n, m.value, mn.value
+
+
+def footprints():
+    """[wait entered, wait passed, pack started, sum done, wait timed out] sequence numbers (TBV_KWAIT=1)."""
+    buf = (ctypes.c_ulonglong * 5)()
+    _lib.tbv_emu_footprints(buf)
+    return list(buf)
 
 
 def tag_counts():

@@ -240,3 +240,29 @@ def test_latency_and_phase_breakdown(orc, capfd):
         tbv.hist()
         assert " B~ :" not in capfd.readouterr().err                      # the dump reset the histogram
         tbv.stage_peer_repeat(None)
+
+
+@pytest.mark.parametrize("name", ["bf16", "f16", "f32"])
+def test_nan_and_inf_propagation(orc, name):
+    """NaN in -> NaN out, Inf - Inf -> NaN, Inf + finite -> Inf: the positions must agree with the oracle and all
+    non-NaN results must match it bit for bit.  Which NaN comes out (payload, sign) is not pinned."""
+    dt = DT[name]
+    n = 4096
+    a = synth.normal(3, n); b = synth.normal(4, n)
+    a[::7] = np.inf; b[::11] = -np.inf; a[5::13] = np.nan; b[9::17] = np.nan; a[::77] = -np.inf
+    ta, tb = dev(a, dt), dev(b, dt)
+    with session(rails=1, cap=1 << 20) as tbv:
+        out = torch.empty_like(ta)
+        tbv.stage_peer(tb)
+        assert tbv.all_reduce(ta, out)
+        torch.cuda.synchronize()
+        want = oracle_sum(orc, ta, tb)
+        nan = torch.isnan(want)
+        assert int(nan.sum()) > 400 and torch.equal(torch.isnan(out.cpu()), nan)
+        if name == "f32":
+            g, w = out.cpu().numpy().view(np.uint32), want.numpy().view(np.uint32)
+        else:
+            g, w = bits_np(out), bits_np(want)
+        keep = ~nan.numpy()
+        assert np.array_equal(g[keep], w[keep])
+        assert int(torch.isinf(out).sum()) > 500

@@ -135,6 +135,27 @@ def test_watchdog_releases_gpu_and_error_is_sticky(orc):
         tbv.withhold(0, 0)
 
 
+def test_watchdog_on_missing_pack_completion(orc):
+    """The pack kernel of call 2 never raises its completion word (forced from the host): the progress
+    threads give up after TBV_WDOG, set the error flag and still release the GPU."""
+    with session(rails=2, cap=1 << 20, TBV_WDOG=1, TBV_FUSEWAIT=0) as tbv:
+        a = dev(synth.normal(1, 1 << 18), torch.bfloat16); p = dev(synth.normal(2, 1 << 18), torch.bfloat16)
+        out = torch.empty_like(a)
+        tbv.stage_peer(p); assert tbv.all_reduce(a, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, a + p)
+        tbv.withhold(2, -1)
+        tbv.stage_peer(p)
+        t0 = time.time()
+        assert tbv.all_reduce(a, out)
+        torch.cuda.synchronize()
+        assert 0.8 < time.time() - t0 < 4.0
+        assert tbv.err()
+        with pytest.raises(RuntimeError):
+            tbv.all_reduce(a, out)
+        tbv.withhold(0, 0)
+
+
 # ---------------------------------------------------------------- every mode gives the same bits
 
 MODES = {
@@ -191,6 +212,10 @@ def test_modes_bit_exact(orc, mode):
         torch.cuda.synchronize()
         assert torch.equal(out, a + a)
         assert not tbv.err()
+        if mode == "kwait":
+            torch.cuda.synchronize()
+            last = tbv.seq()
+            assert tbv.footprints() == [last, last, last, last, 0]      # wait in, wait out, pack, sum done; no timeout
         if mode == "tag":
             checks, bad_plain, bad_sys = tbv.tag_counts()
             assert checks == k + 1 and bad_plain == 0 and bad_sys == 0
