@@ -433,8 +433,8 @@ int configure(const char* devs, size_t cap)
     G.fuse = geti("TBV_FUSE", 0);
     // uncached bounce: waves only drain their stores; cached bounce: block leader writes the L2 back
     G.packsig = geti("TBV_PACKSIG", (G.uncached & 1) ? 0 : 1);
-    // messages that travel on one rail poll their flag inside the sum kernel by default
-    G.fusewait_max = getz("TBV_FUSEWAIT", G.rail1max);
+    // decode-size messages (up to 1 MiB: batch 128 x hidden 4096 x 2 B is 1 MiB) poll their flag inside the kernel
+    G.fusewait_max = getz("TBV_FUSEWAIT", (size_t)1 << 20);
     G.defer = geti("TBV_DEFERSIG", 1);
     G.onekernel = geti("TBV_ONEKERNEL", 1);
     { const char* e = getenv("TBV_WIRE");

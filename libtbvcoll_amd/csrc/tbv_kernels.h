@@ -67,7 +67,7 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullpt
 hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 // A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
 // blocks of 1024 lanes, one 16-byte vector per lane.
-static constexpr int kSmallCallMaxBlocks = 16;
+static constexpr int kSmallCallMaxBlocks = 64;       // 1 MiB; 64 x 16 waves = an eighth of the GPU's wave slots
 int small_call_blocks(size_t nbytes);
 hipError_t launch_small_call(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_waitflag(const unsigned long long* flag, unsigned long long seq,

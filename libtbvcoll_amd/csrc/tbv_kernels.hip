@@ -59,6 +59,10 @@ __device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_typ
 static constexpr int kThreads = 256;        // 4 wavefronts of 64
 static constexpr int kMaxSmallThreads = 1024;
 static constexpr int kMaxGrid = 256 * 8;     // 256 CUs, up to 8 resident blocks each
+// A kernel that waits for the flag inside holds its wave slots while it waits.  Whatever has to
+// run for the flag to come up (another stream's copy, another library's kernel) needs slots too,
+// so a gated grid is kept to an eighth of the GPU's 8192 wave slots; the blocks loop instead.
+static constexpr int kGatedMaxGrid = 256;
 
 // ---------------------------------------------------------------- arithmetic
 
@@ -483,10 +487,13 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
         s.done = a.done; s.done_arrive = a.done_arrive;
         s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
         s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
-        return launch_step<false, true>(a.dtype, s, geom_for(a.nbytes), st, t);
+        Geom g = geom_for(a.nbytes);
+        if (a.wait_flag && g.grid > kGatedMaxGrid) g.grid = kGatedMaxGrid;
+        return launch_step<false, true>(a.dtype, s, g, st, t);
     }
     size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
     int grid = (int)((n + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid; if (grid < 1) grid = 1;
+    if (a.wait_flag && grid > kGatedMaxGrid) grid = kGatedMaxGrid;
     switch (a.dtype) {
         case 0: return launch1(k_sum_narrow<0>, grid, kThreads, st, t, a);
         case 1: return launch1(k_sum_narrow<1>, grid, kThreads, st, t, a);

@@ -52,9 +52,9 @@ def test_exact(orc, mode):
 
 # ---------------------------------------------------------------- counterpart of step4/test_stress.py
 
-@pytest.mark.parametrize("name,nb,rails", [("bf16", 57344, 2), ("f16", 229376, 2), ("f32", 8192, 1)])
-def test_stress_back_to_back(orc, name, nb, rails):
-    iters = 2000
+@pytest.mark.parametrize("name,nb,rails,iters", [("bf16", 57344, 2, 2000), ("f16", 229376, 2, 2000), ("f32", 8192, 1, 2000),
+                                                 ("bf16", 8192, 1, 10000)])     # last: the decode config, NSLOT=4, CAP=8 KB
+def test_stress_back_to_back(orc, name, nb, rails, iters):
     dt = DT[name]
     numel = nb // torch.tensor([], dtype=dt).element_size()
     with session(rails=rails, cap=nb, TBV_NSLOT=4) as tbv:

@@ -170,7 +170,7 @@ MODES = {
     "stream_gate_only": {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0, "TBV_ONEKERNEL": 0},
     "no_defer": {"TBV_DEFERSIG": 0},
     "two_kernels": {"TBV_ONEKERNEL": 0},
-    "one_kernel_256k": {"TBV_FUSEWAIT": 262144},
+    "fusewait_96k": {"TBV_FUSEWAIT": 98304},
     "fusewait_no_defer": {"TBV_FUSEWAIT": 1 << 30, "TBV_DEFERSIG": 0},
     "block512": {"TBV_BLOCK": 512, "TBV_UNROLL": 2, "TBV_GRIDCAP": 256},
     "host_wire": {"TBV_WIRE": "host"},
