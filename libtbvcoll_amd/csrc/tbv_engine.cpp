@@ -579,16 +579,16 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         if (G.gpusig) {
             const bool can_fuse = G.fuse && c->resident && sum_out && !G.tag &&
                                   !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
-            // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
-            // When the next kernel on the stream is one of ours and will not wait behind a stream gate
-            // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
-            // completion word alone and that next kernel raises it first thing.
             // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
             // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
             const bool one_kernel = G.onekernel && !can_fuse && sum_out && !G.tag && G.kwait != 1 && G.can_wait_value &&
                                     !(G.railsum && c->R > 1) && nbytes <= G.fusewait_max &&
                                     tbv::small_call_blocks(nbytes) <= tbv::kSmallCallMaxBlocks &&
                                     !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
+            // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
+            // When the next kernel on the stream is one of ours and will not wait behind a stream gate
+            // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
+            // completion word alone and that next kernel raises it first thing.
             const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
             c->deferred = G.defer && !can_fuse && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
