@@ -175,6 +175,9 @@ def main():
 
     import torch
     from libtbvcoll_amd import synth, tbvcoll as tbv
+    if not os.path.exists(os.path.join(ROOT, "libtbvcoll_amd", "libtbvcoll.so")):       # load what is built; build only if nothing is
+        import __graft_entry__
+        __graft_entry__.build()
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the data path has no CPU fallback", file=sys.stderr)
         sys.exit(3)

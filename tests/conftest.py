@@ -11,6 +11,12 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # load what is built; build only if nothing is (hipcc cross-compiles gfx950 without a GPU)
+    import subprocess
+    if not os.path.exists(os.path.join(ROOT, "libtbvcoll_amd", "libtbvcoll.so")):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "libtbvcoll_amd", "csrc")], check=True, stdout=subprocess.DEVNULL)
+    if not (os.path.exists(os.path.join(ROOT, "oracle", "liborc.so")) and os.path.exists(os.path.join(ROOT, "oracle", "libhiphdr.so"))):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True, stdout=subprocess.DEVNULL)
 
 
 @pytest.fixture(scope="session")
