@@ -797,10 +797,10 @@ int drain_rails()
 
 // ========================================================================== C ABI, part 1
 
-extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_t cap)
+static void teardown();
+
+static int init_impl(int rank, const char* devs, size_t cap)
 {
-    (void)peer_ip; (void)port;
-    if (G.inited) return 0;
     if (configure(devs, cap) != 0) return -1;
     G.rank = rank;
     if (hipGetDevice(&G.device) != hipSuccess) FAIL("no HIP device");
@@ -859,6 +859,15 @@ extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int 
     LOGF("  small calls (<= %zu B) in one kernel: %s", G.fusewait_max, G.onekernel ? "yes" : "no");
     LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
     return 0;
+}
+
+extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_t cap)
+{
+    (void)peer_ip; (void)port;
+    if (G.inited) return 0;
+    const int rc = init_impl(rank, devs, cap);
+    if (rc != 0) teardown();               // a failed initialisation leaves nothing allocated and no thread running
+    return rc;
 }
 
 extern "C" int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype, void* stream)
@@ -1156,14 +1165,20 @@ extern "C" void tbv_emu_tag_counts(unsigned long long* checks, unsigned long lon
 extern "C" void tbv_emu_shutdown(void)
 {
     if (!G.inited) { G.configured = 0; return; }
+    teardown();
+}
+
+// Releases whatever exists, whether or not initialisation completed.
+static void teardown()
+{
     // let the GPU finish what is queued (flags are raised even after an error), then stop the threads
     (void)hipDeviceSynchronize();
     tbv_ar_fini();
-    for (int r = 0; r < G.R; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
+    for (int r = 0; r < MAXRAIL; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
     for (auto& o : G.owned) (void)hipFree(o.first);
     G.owned.clear();
     G.stream_wire.clear();
-    for (int i = 0; i < G.nslot; i++) if (G.ev[i]) { (void)hipEventDestroy(G.ev[i]); G.ev[i] = nullptr; }
+    for (int i = 0; i < MAXSLOT; i++) if (G.ev[i]) { (void)hipEventDestroy(G.ev[i]); G.ev[i] = nullptr; }
     free_slab(G.sendbase, g_uc_send); G.sendbase = nullptr;
     free_slab(G.recvbase, g_uc_recv); G.recvbase = nullptr;
     if (G.hostwords) { (void)hipHostFree(G.hostwords); G.hostwords = nullptr; }

@@ -90,6 +90,15 @@ def test_rail_plan_against_oracle(orc, rails, env):
         lib.tbv_emu_shutdown()
 
 
+def test_failed_init_returns_minus_one_and_leaves_nothing_behind():
+    lib = tbvcoll.load()
+    lib.tbv_emu_shutdown()
+    assert lib.tbv_ar_init(0, b"a,b,c,d,e", b"", 18995, 4096) == -1           # five rails: refused before any allocation
+    assert lib.tbv_ar_cap() >= 0 and lib.tbv_ar_err() == 0
+    assert lib.tbv_ar_allreduce(None, None, 16, 0, None) == -1               # still not initialised
+    lib.tbv_emu_shutdown()
+
+
 def test_configure_rejects_bad_rail_counts():
     lib = tbvcoll.load()
     lib.tbv_emu_shutdown()
