@@ -5,8 +5,6 @@
 #include <hsa/hsa_ext_amd.h>
 #include <time.h>
 
-#include <mutex>
-
 namespace tbv {
 namespace {
 
@@ -113,10 +111,6 @@ int dma_copy(int lane, void* dst, DmaSide dst_side, const void* src, DmaSide src
 {
     if (!ready || lane < 0 || lane >= nlanes) return -1;
     if (n == 0) return 0;
-    // One transfer at a time, start to completion: a host-to-device transfer issued from one thread
-    // while another thread's device-to-device transfer was in flight never completed on ROCm 7.0/7.2.
-    static std::mutex one_at_a_time;
-    std::lock_guard<std::mutex> lk(one_at_a_time);
     const hsa_agent_t da = dst_side == DMA_HOST ? host_agent_of(dst) : gpu;
     const hsa_agent_t sa = src_side == DMA_HOST ? host_agent_of(src) : gpu;
     api.signal_store_relaxed(sig[lane], 1);

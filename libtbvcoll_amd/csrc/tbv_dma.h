@@ -17,7 +17,10 @@ void dma_fini();
 bool dma_ready();
 
 // Blocking copy of n bytes on lane `lane`'s signal; each lane is used by one
-// thread at a time.  Transfers of different lanes are serialised internally.  Returns 0, -1 on an engine error, -2 when `timeout_s` passed.
+// thread at a time; lanes are independent.  A transfer that reads host memory
+// uses the runtime's host-to-device engine, which works in order: it queues
+// behind every host-to-device copy the process has issued before, including ones
+// that wait for a stream.  Returns 0, -1 on an engine error, -2 when `timeout_s` passed.
 int dma_copy(int lane, void* dst, DmaSide dst_side, const void* src, DmaSide src_side, size_t n, double timeout_s);
 
 }  // namespace tbv
