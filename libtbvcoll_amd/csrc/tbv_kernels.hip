@@ -184,7 +184,9 @@ __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsign
         const unsigned long long t0 = wall_clock64();
         if (blockIdx.x == 0 || !relay) {
             if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_IN, seq);
-            while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
+            // relaxed polls: an acquire load in the loop would invalidate the caches on every iteration, for this
+            // kernel and for whatever is writing the payload; one acquire fence follows the barrier below
+            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
                 __builtin_amdgcn_s_sleep(1);
                 if (wall_clock64() - t0 > limit) {
                     if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
@@ -194,7 +196,7 @@ __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsign
             if (relay) __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_OUT, seq);
         } else {
-            while (__hip_atomic_load(relay, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < seq) {
+            while (__hip_atomic_load(relay, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < seq) {
                 __builtin_amdgcn_s_sleep(2);
                 if (wall_clock64() - t0 > limit + limit / 8 + 1000000ull) break;
             }
