@@ -253,3 +253,18 @@ def test_whole_step_threaded_equals_single(orc):
     b4, o4 = orc.reduce_copy(2, a, b, 4)
     assert np.array_equal(b1, a) and np.array_equal(b4, a)
     assert np.array_equal(o1, o4) and np.array_equal(o1, orc.sum_bits(2, a, b))
+
+
+def test_reference_known_answer_one_plus_two(orc):
+    """The known answer the reference's own programs check: rank 0 holds 1.0, rank 1 holds 2.0, every
+    element of the result is 3.0 (step4/allreduce2.cpp:203-206, step4/allreduce_mr.cpp:222-225,
+    step4/test_tbvcoll.py:51-55,67-69)."""
+    n = 1024
+    for code, one, two, three in ((0, 0x3F800000, 0x40000000, 0x40400000), (1, 0x3C00, 0x4000, 0x4200), (2, 0x3F80, 0x4000, 0x4040)):
+        dt = np.uint32 if code == 0 else np.uint16
+        a = np.full(n, one, dtype=dt); b = np.full(n, two, dtype=dt)
+        if code == 0:
+            got = orc.sum_bits(0, a.view(np.float32), b.view(np.float32)).view(np.uint32)
+        else:
+            got = orc.sum_bits(code, a, b)
+        assert np.array_equal(got, np.full(n, three, dtype=dt))
