@@ -131,7 +131,7 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
     os.environ.pop("TBV_ONEKERNEL", None)
     return {"p50_us": round(pct(lat, 0.50), 2), "p99_us": round(pct(lat, 0.99), 2), "min_us": round(min(lat), 2),
             "samples": len(lat), "us_per_call_wall": round(wall / iters * 1e6, 2), "bit_exact": ok,
-            "gate": "one kernel per call: pack, completion word, flag poll, sum (library default for one-rail sizes)" if fusewait
+            "gate": "one kernel per call: pack, completion word, flag poll, sum (library default up to 1 MiB)" if fusewait
             else "pack kernel, hipStreamWaitValue64, sum kernel (TBV_FUSEWAIT=0 TBV_DEFERSIG=0 TBV_ONEKERNEL=0)",
             "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word"}
 
