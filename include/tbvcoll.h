@@ -82,6 +82,7 @@ void tbv_ar_fini(void);
  * rail's fragment of the peer payload into the receive slot on a side stream and
  * then raises a 64-bit arrival word on that stream, which is the signal the
  * immediate's completion gave.  None of these symbols exist in the reference.
+ * Like tbv_ar_allreduce they are to be called from the one caller thread.
  */
 
 /* Queue the peer's payload for the next call that has none yet (FIFO, one entry per
