@@ -2,25 +2,33 @@
 """Benchmark of the all-reduce data path on one MI355X.
 
 A step is one tbv_ar_allreduce call through the C ABI on the 16 MiB bf16 prefill
-workload with the peer's payload already resident in the receive slots: pack copy
-into the uncached send bounce (with completion word), the 64-bit flag wait, the
-sum kernel into the output.  Algorithmic bytes per step are 5N (pack 2N + sum 3N).
+workload with the peer's payload already in the receive slots: the local tensor is
+copied into the uncached send bounce (completion word raised), and local + received
+is written to the output.  Algorithmic bytes per step are 5N (pack 2N + sum 3N).
 
-Prints ONE JSON line.  Besides the throughput it carries
-  roofline      the sum kernel (the dominant one) against the 8 TB/s HBM peak,
-                timed with HIP events recorded on the caller's stream around every
-                launch of a second pass of the same steps;
-  cpu_baseline  the CPU oracle's restatement of the same step on the host cores;
-  cache_cold    the same step with buffers rotated beyond the Infinity Cache;
-  decode_latency  p50/p99 of (flag raised -> sum complete) for the 8 KB decode
-                workload, 10,000 back-to-back calls: library default (flag polled
-                inside the sum kernel) and, as decode_latency_stream_gate, gated by
-                hipStreamWaitValue64 as the reference does.
+The headline (`value`, `roofline`) is the HBM-bound form of that step: 16 ring slots
+and 12 rotating local/output tensors, 896 MiB touched in turn, so every operand comes
+from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also carries
+
+  long_run         the same leg over 2000 steps when --steps is small
+  cold_two_launches, cold_fused_4N   the same cold step as pack kernel + sum kernel, and
+                   as one kernel that reads the local tensor once (4N)
+  resident         the step with everything it touches resident in the Infinity Cache
+                   (4 slots, one local/output tensor): a cache figure, labelled so
+  achievable       what plain read / write / copy kernels reach on this GPU (1 GiB
+                   buffers, and 16 MiB cache-cold), and the launch-to-launch floor
+  decode_latency   p50/p99 of (flag raised -> sum complete) for the 8 KB decode
+                   workload, 10,000 back-to-back calls: library default (one kernel per
+                   call) and, as decode_latency_stream_gate, the reference's sequence
+                   pack kernel, hipStreamWaitValue64, sum kernel
+  pipeline_64MiB_fp16  64 MiB fp16 as 16 chunks of 4 MiB over 2 rails x 4 slots
+  cpu_baseline     the CPU oracle's restatement of the same step on the host cores.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -28,12 +36,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12                      # MI355X HBM3E, bytes/s
-# Bytes the sum kernel moves between L2 and memory per 16 MiB launch, from rocprofv3 counter runs of this
-# command (profiles/prefill16MiB_pmc_fetch_write.txt): FETCH_SIZE 16407.5 KiB x 1.9972 (what the counter
-# reads for a plain 16 MiB copy, 8203.5 KiB for 16384 KiB) + WRITE_SIZE 16384.0 KiB x 1.0.
-SUM_TRAFFIC_BYTES = int((16407.5 * (16384.0 / 8203.5) + 16384.0) * 1024)
 N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
+COLD_NSLOT, COLD_NBUF = 16, 12         # 2 x 16 x 16 MiB of rings + 2 x 12 x 16 MiB of tensors = 896 MiB
+TRAFFIC_FILE = os.path.join("profiles", "prefill16MiB_cold_pmc_fetch_write.txt")
+TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL")
 
 
 def pct(xs, q):
@@ -41,20 +48,42 @@ def pct(xs, q):
     return xs[min(len(xs) - 1, int(q * len(xs)))]
 
 
-def run_prefill(tbv, torch, synth, st, steps, warmup, fuse, nslot=4, nbuf=1):
-    """nslot=4, nbuf=1 is the workload as specified (everything a step touches, 160 MiB, fits the 256 MB
-    Infinity Cache).  nslot=16 with nbuf=12 rotating local/out tensors touches 896 MiB in turn, so every
-    step's operands come from HBM: the cache-cold figure."""
+def traffic_from_profile(kernel):
+    """HBM-side bytes per launch of `kernel` as the committed counter summary states them
+    (a line `TRAFFIC kernel=<name> bytes_per_launch=<n>`); None when the file has no such line."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            for ln in f:
+                m = re.match(r"\s*TRAFFIC kernel=(\S+) bytes_per_launch=(\d+)", ln)
+                if m and m.group(1) == kernel:
+                    return int(m.group(2))
+    except OSError:
+        pass
+    return None
+
+
+def own_warmup(warmup, nslot, nbuf):
+    """Untimed steps before the clock: at least two full periods of the (tensor, slot) rotation."""
+    import math
+    return max(warmup, 2 * math.lcm(nslot, nbuf), 48)
+
+
+def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0):
+    """`steps` timed calls after `warmup` untimed ones (never fewer than two turns of every rotating tensor and
+    ring slot, so no buffer is touched for the first time inside the clock), then an optional long run, then a
+    pass of the same steps with the dispatch timestamps of every kernel launch."""
     n = N_PREFILL
+    for k in TUNING_KEYS:
+        os.environ.pop(k, None)
     os.environ["TBV_NSLOT"] = str(nslot)
-    os.environ["TBV_FUSE"] = "1" if fuse else "0"
+    for k, v in env:
+        os.environ[k] = str(v)
     tbv.shutdown()
     tbv.init(0, "rail0,rail1", "", cap_bytes=n)
     a = torch.from_numpy(synth.prefill_activations(100, n // 2)).to(torch.bfloat16).cuda()
     b = torch.from_numpy(synth.prefill_activations(101, n // 2)).to(torch.bfloat16).cuda()
-    out = torch.empty_like(a)
     locs = [a] + [a.clone() for _ in range(nbuf - 1)]
-    outs = [out] + [torch.empty_like(a) for _ in range(nbuf - 1)]
+    outs = [torch.empty_like(a) for _ in range(nbuf)]
     fn = tbv.raw_fn()
     ps = ctypes.c_void_p(st.cuda_stream)
     ptrs = [(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(o.data_ptr())) for x, o in zip(locs, outs)]
@@ -68,20 +97,35 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, fuse, nslot=4, nbuf=1):
         if rc != 0:
             raise RuntimeError(f"tbv_ar_allreduce rc={rc}")
 
-    for _ in range(warmup):
+    def timed(k):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(k):
+            step()
+        while not st.query():          # poll, so that the synchronize below returns at once instead of after a sleep
+            pass
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    for _ in range(own_warmup(warmup, nslot, nbuf)):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
+    tbv.stats4()                       # drop what the warm-up (and the first call's stream probe) accumulated
+    wall = timed(steps)
+    tbv.stats4()
+    long_wall = timed(long_steps) if long_steps else None
+    # host cost of one call, from a burst short enough never to wait for room in the ring
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    tbv.stats4()
+    for _ in range(min(nslot - 1, 12)):
+        step()
+    enq = tbv.stats4()[3]
+    torch.cuda.synchronize()
     want = a + b
     ok = all(bool(torch.equal(o, want)) for o in outs)    # the timed path computed the sum, bit for bit
-    enq = tbv.stats4()[3]
+    tbv.stats4()
 
-    # second pass of the same steps with an event pair around every kernel launch
-    ksteps = min(steps, 1000)
+    ksteps = max(min(steps, 1000), 240)
     tbv.kernel_timing(True)
     for _ in range(ksteps):
         step()
@@ -91,14 +135,43 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, fuse, nslot=4, nbuf=1):
     torch.cuda.synchronize()
     err = tbv.err()
     tbv.shutdown()
-    return {"wall": wall, "ok": ok and not err, "enq_us": enq, "pack_us": pack_us, "pack_min_us": pack_min, "n_pack": n_pack,
-            "sum_us": sum_us, "sum_min_us": sum_min, "n_sum": n_sum}
+    for k, _ in env:
+        os.environ.pop(k, None)
+    return {"wall": wall, "steps": steps, "long_wall": long_wall, "long_steps": long_steps, "ok": ok and not err, "enq_us": enq,
+            "pack_us": pack_us, "pack_min_us": pack_min, "n_pack": n_pack, "sum_us": sum_us, "sum_min_us": sum_min, "n_sum": n_sum}
+
+
+def kernel_roofline(nbytes, us, min_us, launches, ceiling_gbps=None):
+    if not us or us <= 0:
+        return None
+    gbps = nbytes / (us * 1e-6) / 1e9
+    r = {"algorithmic_bytes": nbytes, "avg_launch_us": round(us, 3), "min_launch_us": round(min_us, 3), "launches": launches,
+         "achieved": round(gbps, 1), "unit": "GB/s", "frac": round(gbps * 1e9 / HBM_PEAK, 4)}
+    if ceiling_gbps:
+        r["frac_of_measured_copy_ceiling"] = round(gbps / ceiling_gbps, 4)
+    return r
+
+
+def run_achievable(tbv):
+    """Plain streaming kernels shipped in the library: the denominators this GPU really offers."""
+    gib = 1 << 30
+    out = {"what": "in-tree read / write / copy kernels (16-byte vectors, 256-lane blocks), dispatch timestamps; 1 GiB buffers, "
+                   "and 16 MiB launches walking a 1 GiB pool (cache-cold)"}
+    for name, kind, nbytes, pool, reps, mult in (("read_1GiB", 0, gib, gib, 10, 1), ("write_1GiB", 1, gib, gib, 10, 1),
+                                                 ("copy_1GiB", 2, gib, gib, 10, 2), ("copy_plain_1GiB", 3, gib, gib, 10, 2),
+                                                 ("copy_16MiB_cold", 2, N_PREFILL, gib, 120, 2), ("read_16MiB_cold", 0, N_PREFILL, gib, 120, 1)):
+        mean, mn = tbv.hbm_probe(kind, nbytes, pool, reps)
+        out[name] = {"GBps": round(mult * nbytes / (mean * 1e-6) / 1e9, 1), "avg_us": round(mean, 2), "min_us": round(mn, 2),
+                     "frac_of_peak": round(mult * nbytes / (mean * 1e-6) / HBM_PEAK, 4)}
+    out["empty_kernel_launch_to_launch_us"] = round(tbv.launch_floor(2000), 2)
+    return out
 
 
 def run_decode(tbv, torch, synth, st, iters, fusewait):
     n = N_DECODE
+    for k in TUNING_KEYS:
+        os.environ.pop(k, None)
     os.environ["TBV_NSLOT"] = "4"
-    os.environ["TBV_FUSE"] = "0"
     os.environ["TBV_FUSEWAIT"] = str(n) if fusewait else "0"
     os.environ["TBV_DEFERSIG"] = "1" if fusewait else "0"
     os.environ["TBV_ONEKERNEL"] = "1" if fusewait else "0"
@@ -114,6 +187,7 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
             tbv.stage_peer(peers[it % npeer]); tbv.all_reduce(locs[it % npeer], outs[it % npeer])
         torch.cuda.synchronize()
         tbv.latencies()
+        tbv.stats4()
         t0 = time.perf_counter()
         for it in range(iters):
             k = it % npeer
@@ -122,18 +196,55 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
                 raise RuntimeError("decode call not handled")
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
+    _, _, post, enq, _ = tbv.stats4()
     lat = tbv.latencies()
     ok = all(bool(torch.equal(outs[k], locs[k] + peers[k])) for k in range(npeer)) and not tbv.err()
     tbv.latency_probe(False)
     tbv.shutdown()
-    os.environ.pop("TBV_FUSEWAIT", None)
-    os.environ.pop("TBV_DEFERSIG", None)
-    os.environ.pop("TBV_ONEKERNEL", None)
+    for k in TUNING_KEYS:
+        os.environ.pop(k, None)
     return {"p50_us": round(pct(lat, 0.50), 2), "p99_us": round(pct(lat, 0.99), 2), "min_us": round(min(lat), 2),
             "samples": len(lat), "us_per_call_wall": round(wall / iters * 1e6, 2), "bit_exact": ok,
+            "host_enqueue_us": round(enq, 2), "host_post_us": round(post, 2),
             "gate": "one kernel per call: pack, completion word, flag poll, sum (library default up to 1 MiB)" if fusewait
             else "pack kernel, hipStreamWaitValue64, sum kernel (TBV_FUSEWAIT=0 TBV_DEFERSIG=0 TBV_ONEKERNEL=0)",
-            "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word"}
+            "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word; "
+                        "host_enqueue_us is the time inside tbv_ar_allreduce per call, host_post_us its last launch"}
+
+
+def run_pipeline(tbv, torch, synth, st, reps=20):
+    """64 MiB fp16 as 16 chunks of CAP = 4 MiB over 2 rails x 4 slots, each (chunk, rail) fragment deposited by a
+    side-stream copy and signalled by a 64-bit flag; three packs ahead, so sums overlap arrivals."""
+    cap, nchunks = 4 << 20, 16
+    numel = nchunks * cap // 2
+    for k in TUNING_KEYS:
+        os.environ.pop(k, None)
+    os.environ["TBV_NSLOT"] = "4"
+    tbv.shutdown()
+    tbv.init(0, "rail0,rail1", "", cap_bytes=cap)
+    a = torch.from_numpy(synth.normal(41, numel)).to(torch.float16).cuda()
+    p = torch.from_numpy(synth.normal(42, numel)).to(torch.float16).cuda()
+    out = torch.empty_like(a)
+    per = cap // 2
+    times = []
+    with torch.cuda.stream(st):
+        for r in range(reps + 3):
+            for c in range(nchunks):
+                tbv.stage_peer(p[c * per:(c + 1) * per])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            tbv.all_reduce_chunked(a, out)
+            torch.cuda.synchronize()
+            if r >= 3:
+                times.append(time.perf_counter() - t0)
+    ok = bool(torch.equal(out, a + p)) and not tbv.err()
+    tbv.shutdown()
+    os.environ.pop("TBV_NSLOT", None)
+    med = pct(times, 0.5)
+    return {"us": round(med * 1e6, 1), "min_us": round(min(times) * 1e6, 1), "GBps_5N": round(5 * numel * 2 / med / 1e9, 1),
+            "bit_exact": ok, "reps": reps,
+            "what": "tbv_ar_allreduce_chunked, 16 x 4 MiB fp16, 2 rails x NSLOT 4, every fragment through the emulated wire; "
+                    "host clock from the call to the stream's completion, median"}
 
 
 def run_cpu_baseline(torch, synth):
@@ -161,17 +272,19 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
-    ap.add_argument("--fuse", type=int, default=0, help="1: pack+sum in one kernel when the peer is resident (4N)")
+    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,cpu",
+                    help="comma list of the extra legs to run beside the headline (cold) leg")
+    ap.add_argument("--headline-env", default="", help="TBV_X=v,... applied to the headline leg (for profiling one variant)")
+    ap.add_argument("--rotate", default=f"{COLD_NSLOT},{COLD_NBUF}",
+                    help="ring slots, rotating local/output tensors of the headline leg (4,1 = the cache-resident shape; for experiments)")
     ap.add_argument("--calibrate-copy", type=int, default=0,
                     help="also run this many plain 16 MiB device copies (known 16 MiB read + 16 MiB written), "
                          "so a counter run of this command holds a kernel of known traffic to scale by")
-    ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--skip-decode", action="store_true")
-    ap.add_argument("--skip-cold", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1", file=sys.stderr)
         sys.exit(2)
+    legs = set(x for x in args.legs.split(",") if x)
 
     import torch
     from libtbvcoll_amd import synth, tbvcoll as tbv
@@ -187,54 +300,91 @@ def main():
     # caller's stream and a rail's side stream on the same hardware queue (the engine would then fall back
     # to its slower host wire, which only matters for the emulated peer, not for the timed kernels)
     st = torch.cuda.Stream()
-    pre = run_prefill(tbv, torch, synth, st, args.steps, args.warmup, bool(args.fuse))
+    n = N_PREFILL
+    henv = tuple(tuple(kv.split("=", 1)) for kv in args.headline_env.split(",") if kv)
+    fused_headline = dict(henv).get("TBV_FUSE") == "1"
+    two_headline = dict(henv).get("TBV_MERGE") == "0" and not fused_headline
+    long_steps = 2000 if args.steps < 1000 else 0
+    h_nslot, h_nbuf = (int(x) for x in args.rotate.split(","))
+    cold = run_prefill(tbv, torch, synth, st, args.steps, args.warmup, h_nslot, h_nbuf, env=henv, long_steps=long_steps)
     if args.calibrate_copy:
         src = torch.empty(N_PREFILL, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
         for _ in range(args.calibrate_copy):
             dst.copy_(src)
         torch.cuda.synchronize()
-    n = N_PREFILL
-    alg_step = (4 if args.fuse else 5) * n
-    ms = pre["wall"] / args.steps * 1e3
-    dom_bytes = (4 if args.fuse else 3) * n
-    achieved = dom_bytes / (pre["sum_us"] * 1e-6) / 1e9 if pre["sum_us"] > 0 else 0.0
+
+    ach = run_achievable(tbv) if "achievable" in legs else None
+    ceiling = ach["copy_1GiB"]["GBps"] if ach else None
+    alg_step = (4 if fused_headline else 5) * n
+    ms = cold["wall"] / args.steps * 1e3
+    dom_kernel = "sum" if two_headline else ("pack+sum fused" if fused_headline else "pack+sum merged launch")
+    dom_bytes = 3 * n if two_headline else alg_step
+    roof = kernel_roofline(dom_bytes, cold["sum_us"], cold["sum_min_us"], cold["n_sum"], ceiling) or {}
+    traffic_kernel = "k_step_sum" if two_headline else ("k_step_pack_sum" if fused_headline else "k_merged")
+    traffic = traffic_from_profile(traffic_kernel)
     line = {
         "metric": "reduce-copy GB/s at 16MB bf16", "value": round(alg_step / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "prefill all-reduce step, bf16 [2048x4096] = 16 MiB local + peer payload resident in the "
-                               "receive slots; values N(0,0.02^2) with 0.1% outliers at +-8",
-                   "step": "pack+sum fused (4N)" if args.fuse else "pack 2N + flag wait + sum 3N = 5N",
-                   "nslot": 4, "rails": 2, "accumulate": "f32, round to nearest even", "bit_exact_vs_torch_add": pre["ok"],
-                   "residency": "everything a step touches (local 16 + bounce ring 64 + receive ring 64 + out 16 MiB) fits the "
-                                "256 MB Infinity Cache; cache_cold in this line is the same step with the buffers rotated beyond it",
-                   "host_enqueue_us_per_call": round(pre["enq_us"], 2)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None if args.fuse else SUM_TRAFFIC_BYTES,
-                     "kernel": "pack+sum" if args.fuse else "sum", "algorithmic_bytes": dom_bytes,
-                     "avg_launch_us": round(pre["sum_us"], 3), "min_launch_us": round(pre["sum_min_us"], 3),
-                     "launches": pre["n_sum"]},
-        "kernels": {"pack": {"algorithmic_bytes": 2 * n, "avg_launch_us": round(pre["pack_us"], 3),
-                             "min_launch_us": round(pre["pack_min_us"], 3), "launches": pre["n_pack"],
-                             "GBps": round(2 * n / (pre["pack_us"] * 1e-6) / 1e9, 1) if pre["pack_us"] > 0 else None}},
+        "config": {"workload": "prefill all-reduce step, bf16 [2048x4096] = 16 MiB local + peer payload pre-staged in the receive "
+                               "slots; values N(0,0.02^2) with 0.1% outliers at +-8; cache-cold: 16 ring slots and 12 rotating "
+                               "local/output tensors (896 MiB touched in turn, beyond the 256 MB Infinity Cache)",
+                   "step": "one kernel reading the local tensor once (4N)" if fused_headline else
+                           ("pack kernel 2N + sum kernel 3N = 5N" if two_headline else
+                            "pack 2N + sum 3N = 5N in one launch (pack blocks and sum blocks side by side)"),
+                   "frac_of_peak": round(alg_step / (ms * 1e-3) / HBM_PEAK, 4),
+                   "frac_of_measured_copy_ceiling": round(alg_step / (ms * 1e-3) / 1e9 / ceiling, 4) if ceiling else None,
+                   "nslot": h_nslot, "rotating_tensors": h_nbuf, "rails": 2, "accumulate": "f32, round to nearest even", "bit_exact_vs_torch_add": cold["ok"],
+                   "untimed_warmup_steps": own_warmup(args.warmup, h_nslot, h_nbuf),
+                   "host_enqueue_us_per_call": round(cold["enq_us"], 2), "headline_env": dict(henv)},
+        "roofline": dict({"bound": "hbm", "kernel": dom_kernel, "peak": HBM_PEAK / 1e9}, **roof,
+                         traffic=traffic, traffic_source=(TRAFFIC_FILE if traffic else None),
+                         timing="dispatch timestamps of every launch in a second pass of the same steps (per-launch events "
+                                "inside the timed region would slow it)"),
     }
-    if not args.skip_cold:
-        cold = run_prefill(tbv, torch, synth, st, min(args.steps, 1000), min(args.warmup, 100), bool(args.fuse), nslot=16, nbuf=12)
-        cms = cold["wall"] / min(args.steps, 1000) * 1e3
-        line["cache_cold"] = {"what": "same step with NSLOT=16 and 12 rotating local/out tensors (896 MiB touched in turn, "
-                                      "beyond the 256 MB Infinity Cache)",
-                              "value": round(alg_step / (cms * 1e-3) / 1e9, 1), "unit": "GB/s", "ms_per_step": round(cms, 5),
-                              "sum_avg_us": round(cold["sum_us"], 3), "pack_avg_us": round(cold["pack_us"], 3),
-                              "sum_frac_of_peak": round(dom_bytes / (cold["sum_us"] * 1e-6) / HBM_PEAK, 4) if cold["sum_us"] else None,
-                              "bit_exact": cold["ok"]}
-    if not args.skip_decode:
+    if two_headline:
+        line["kernels"] = {"pack": kernel_roofline(2 * n, cold["pack_us"], cold["pack_min_us"], cold["n_pack"], ceiling)}
+    if cold["long_wall"]:
+        lms = cold["long_wall"] / cold["long_steps"] * 1e3
+        line["long_run"] = {"steps": cold["long_steps"], "ms_per_step": round(lms, 5), "value": round(alg_step / (lms * 1e-3) / 1e9, 1),
+                            "unit": "GB/s", "frac_of_peak": round(alg_step / (lms * 1e-3) / HBM_PEAK, 4)}
+    if ach:
+        line["achievable"] = ach
+    sub_steps = min(max(args.steps, 500), 2000)
+    if "two" in legs and not two_headline:
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, env=(("TBV_MERGE", 0),))
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_two_launches"] = {"what": "the same cache-cold step as a pack kernel then a sum kernel (TBV_MERGE=0), 5N", "steps": sub_steps,
+                                     "ms_per_step": round(rms, 5), "value": round(5 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                                     "frac_of_peak": round(5 * n / (rms * 1e-3) / HBM_PEAK, 4), "bit_exact": r["ok"],
+                                     "pack": kernel_roofline(2 * n, r["pack_us"], r["pack_min_us"], r["n_pack"], ceiling),
+                                     "sum": kernel_roofline(3 * n, r["sum_us"], r["sum_min_us"], r["n_sum"], ceiling)}
+    if "fused" in legs and not fused_headline:
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, env=(("TBV_FUSE", 1),))
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_fused_4N"] = {"what": "the same cache-cold step as one kernel that reads the local tensor once (TBV_FUSE=1); "
+                                         "its algorithmic bytes are 4N", "steps": sub_steps,
+                                 "ms_per_step": round(rms, 5), "value": round(4 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                                 "frac_of_peak": round(4 * n / (rms * 1e-3) / HBM_PEAK, 4), "bit_exact": r["ok"],
+                                 "kernel": kernel_roofline(4 * n, r["sum_us"], r["sum_min_us"], r["n_sum"], ceiling)}
+    if "resident" in legs:
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, 4, 1)
+        rms = r["wall"] / sub_steps * 1e3
+        line["resident"] = {"bound": "infinity-cache",
+                            "what": "the same step with 4 ring slots and one local/output tensor: everything it touches (160 MiB) stays "
+                                    "in the 256 MB Infinity Cache, so this is a cache figure, not an HBM one",
+                            "steps": sub_steps, "ms_per_step": round(rms, 5), "value": round(5 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                            "bit_exact": r["ok"], "kernel": kernel_roofline(5 * n, r["sum_us"], r["sum_min_us"], r["n_sum"])}
+    if "decode" in legs:
         line["decode_latency"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=True)
         line["decode_latency_stream_gate"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=False)
-    if not args.skip_cpu:
+    if "pipeline" in legs:
+        line["pipeline_64MiB_fp16"] = run_pipeline(tbv, torch, synth, st)
+    if "cpu" in legs:
         line["cpu_baseline"] = run_cpu_baseline(torch, synth)
     print(json.dumps(line), flush=True)
-    if not pre["ok"]:
+    if not cold["ok"]:
         sys.exit(1)
 
 

@@ -35,7 +35,8 @@ extern "C" {
  * count matters (1..4).  peer_ip/port: kept for signature parity, unused by the
  * emulated peer.  cap: largest payload in bytes, rounded up to 4096.
  * Reads TBV_ASYNC, TBV_GPUSIG, TBV_KWAIT, TBV_NSLOT, TBV_CHUNK, TBV_RAIL1MAX,
- * TBV_CPU, TBV_WDOG, TBV_TAG, TBV_UNCACHED once.  Idempotent: a second call
+ * TBV_CPU, TBV_WDOG, TBV_TAG, TBV_UNCACHED (the reference's switches) and this
+ * build's own tuning switches once.  Idempotent: a second call
  * returns 0 and changes nothing.  Returns 0, or -1 after a "[tbvcoll] ..." line
  * on stderr.
  */
@@ -178,6 +179,16 @@ int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, int dtype, vo
  * (into send slot `slot`, with completion signal) or only the sum, on `stream`. */
 int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream);
 int tbv_emu_run_sum(void* out, const void* a, const void* b, size_t nbytes, int dtype, void* stream);
+
+/* What plain streaming kernels reach on this GPU, as measured denominators beside the
+ * published HBM peak (no counterpart in the reference).  tbv_emu_hbm_probe streams
+ * `bytes` per launch (kind 0 read, 1 write, 2 copy with non-temporal accesses, 3 plain
+ * copy) `reps` times through successive windows of a pool of `pool_bytes` that it
+ * allocates and frees itself, and returns the mean and minimum launch duration in
+ * microseconds.  tbv_emu_launch_floor returns the launch-to-launch time of an empty
+ * kernel in one stream.  Both return 0, or -1 on bad arguments or a HIP error. */
+int tbv_emu_hbm_probe(int kind, size_t bytes, size_t pool_bytes, int reps, double* mean_us, double* min_us);
+int tbv_emu_launch_floor(int reps, double* us_per_launch);
 
 #ifdef __cplusplus
 }

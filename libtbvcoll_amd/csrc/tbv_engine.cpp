@@ -83,6 +83,8 @@ struct Engine {
     // configuration
     int configured = 0, inited = 0, rank = 0, R = 0, async = 1, nslot = 8, gpusig = 1, kwait = 0;
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
+    int merge = 1;                            // resident peer: pack and sum blocks in one launch (TBV_MERGE)
+    int streaming = 0;                        // cache-hint profile of the large kernels (TBV_STREAMING, default by ring size)
     size_t cap = 0, stride = 0, rail1max = 96u * 1024u, chunkb = 0, fusewait_max = 0;
     double wdog = 10.0;
     double tick_hz = 1e8;                     // rate of the constant clock the kernels bound their waits with
@@ -444,7 +446,12 @@ int configure(const char* devs, size_t cap)
       G.wr_hwm = (int)std::min<size_t>(96, (size_t)(G.nslot - 1) * per_item); if (G.wr_hwm < 1) G.wr_hwm = 1; }
     G.R = count_rails(devs);
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
-    tbv::set_tuning(geti("TBV_UNROLL", 0), geti("TBV_GRIDCAP", 0), geti("TBV_BLOCK", 0));
+    G.merge = geti("TBV_MERGE", 1);
+    // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
+    // 256 MB Infinity Cache they stay resident from call to call; beyond that every operand streams from HBM.
+    { const size_t working_set = 2 * (size_t)G.nslot * G.stride + 2 * G.cap;
+      G.streaming = geti("TBV_STREAMING", working_set > ((size_t)192 << 20) ? 1 : 0); }
+    tbv::set_tuning(geti("TBV_UNROLL", 0), geti("TBV_GRIDCAP", 0), geti("TBV_BLOCK", 0), G.streaming);
     G.configured = 1;
     return 0;
 }
@@ -585,12 +592,16 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                                     !(G.railsum && c->R > 1) && nbytes <= G.fusewait_max &&
                                     tbv::small_call_blocks(nbytes) <= tbv::kSmallCallMaxBlocks &&
                                     !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
+            // Payload already in place and too large for the one-kernel call: pack blocks and sum blocks in one
+            // launch (a launch costs about 2.4 us of stream time whatever it does).
+            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && sum_out && !G.tag && G.kwait != 1 &&
+                                   G.packsig == 0 && !(G.railsum && c->R > 1) && !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
             // completion word alone and that next kernel raises it first thing.
             const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
-            c->deferred = G.defer && !can_fuse && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
+            c->deferred = G.defer && !can_fuse && !can_merge && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
             pa.pre = take_pending(st);
             // fault injection from the host: this call's pack never raises its completion word
@@ -612,13 +623,14 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (tbv::launch_small_call(pa, sa, st, kt.get()) != hipSuccess) FAIL("one-kernel call launch failed");
                 { std::lock_guard<std::mutex> lk(G.smx); G.t_post += nowt() - tq; }      // the launch that carries the sum
                 c->fused = true;
-            } else if (can_fuse) {
+            } else if (can_fuse || can_merge) {
                 tbv::SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 if (G.probe.load()) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
                 KTimer kt(1);
                 const double tq = nowt();
-                if (tbv::launch_pack_sum(pa, sa, st, kt.get()) != hipSuccess) FAIL("pack+sum kernel launch failed");
+                if ((can_fuse ? tbv::launch_pack_sum(pa, sa, st, kt.get()) : tbv::launch_pack_sum_merged(pa, sa, st, kt.get())) != hipSuccess)
+                    FAIL("pack+sum kernel launch failed");
                 { std::lock_guard<std::mutex> lk(G.smx); G.t_post += nowt() - tq; }
                 c->fused = true;
             } else {
@@ -858,6 +870,8 @@ static int init_impl(int rank, const char* devs, size_t cap)
     LOGF("  wire %s; copy-engine access for the host wire: %s", G.wire_mode == 1 ? "stream" : G.wire_mode == 2 ? "host" : "auto", dma ? "yes" : "no");
     LOGF("  small calls (<= %zu B) in one kernel: %s", G.fusewait_max, G.onekernel ? "yes" : "no");
     LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
+    LOGF("  cache hints: %s profile; early peer above the one-kernel size: %s", G.streaming ? "streaming" : "resident",
+         G.fuse ? "pack+sum fused (4N)" : G.merge ? "pack and sum blocks in one launch" : "two launches");
     return 0;
 }
 

@@ -57,14 +57,20 @@ static constexpr size_t kCounterWords = 16 * 128;
 // Launch geometry is exposed so the host can log and test it.
 int pack_grid(size_t nbytes);
 int sum_grid(size_t nbytes, int dtype);
-// Tuning knobs for experiments: vectors per lane per iteration (1,2,4,8), the grid cap, threads per block.
-void set_tuning(int unroll, int grid_cap, int block);
+// Tuning: vectors per lane per iteration (1,2,4,8; 0 = chosen by the profile), the grid cap and threads per
+// block (0 = defaults), and the cache-hint profile (0 = operands stay cache resident, 1 = streaming from HBM).
+// Every call sets all four.
+void set_tuning(int unroll, int grid_cap, int block, int streaming);
 
 hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullptr);
 // One kernel that does pack (with completion signal) and sum: legal only when the
 // received payload is already in place.
 hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+// Pack and sum in one launch as two sets of blocks (the pack blocks raise the completion word when they
+// are done, the sum blocks read the local tensor themselves); same legality rule as launch_pack_sum, and
+// the bounce must be uncached (sigmode 0).
+hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 // A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
 // blocks of 1024 lanes, one 16-byte vector per lane.
 static constexpr int kSmallCallMaxBlocks = 64;       // 1 MiB; 64 x 16 waves = an eighth of the GPU's wave slots

@@ -20,40 +20,38 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-// Cache hints of the four data streams (1 = non-temporal), as measured on MI355X with
-// the 16 MiB step: the local tensor is read twice (pack, then sum) and the receive
-// slots are re-read every NSLOT calls, so both are left to allocate in the caches;
-// the output is written once and never read here, so it is stored non-temporally and
-// leaves the cache to the operands (sum 7.6 -> 6.6 us); the uncached bounce gains
-// nothing from a hint.  Non-temporal loads of the local tensor cost 2 us per step.
-#ifndef TBV_NT_A
-#define TBV_NT_A 0
-#endif
-#ifndef TBV_NT_B
-#define TBV_NT_B 0
-#endif
-#ifndef TBV_NT_OUT
-#define TBV_NT_OUT 1
-#endif
-#ifndef TBV_NT_BOUNCE
-#define TBV_NT_BOUNCE 0
-#endif
-
-__device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_a(const uint32_t __attribute__((ext_vector_type(4)))* p)
+// Cache hints of the four data streams, two profiles measured on MI355X with the 16 MiB step.
+//
+// Resident profile (STREAM = false): what a step touches stays in the 256 MB Infinity Cache
+// (small rings, the same tensors every step).  The local tensor is read twice (pack, then
+// sum) and the receive slots are re-read every NSLOT calls, so both are left to allocate in
+// the caches; the output is written once and never read here, so it is stored non-temporally
+// and leaves the cache to the operands (sum 7.6 -> 6.6 us); the uncached bounce gets no hint.
+// Non-temporal loads of the local tensor or the receive slot cost 1-2 us per step here.
+//
+// Streaming profile (STREAM = true): the rings are larger than the cache, every operand
+// comes from HBM and nothing written is read again soon.  The receive slot is loaded and
+// the bounce and the output are stored non-temporally; the local tensor keeps ordinary
+// loads because the sum re-reads it a few microseconds after the pack, except in the fused
+// kernel, its only reader (pack + sum
+// 15.98 -> 14.18 us on cache-cold buffers; the same hints cost 0.3 us when everything is
+// cache resident, which is why there are two profiles).
+// ONCE: this kernel is the only reader of the local tensor (pack and sum fused in one body)
+template <bool STREAM, bool ONCE> __device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_a(const uint32_t __attribute__((ext_vector_type(4)))* p)
 {
-    return TBV_NT_A ? __builtin_nontemporal_load(p) : *p;
+    return *p;          // non-temporal here costs about 1 us per 16 MiB even when this kernel is the only reader
 }
-__device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_b(const uint32_t __attribute__((ext_vector_type(4)))* p)
+template <bool STREAM> __device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_b(const uint32_t __attribute__((ext_vector_type(4)))* p)
 {
-    return TBV_NT_B ? __builtin_nontemporal_load(p) : *p;
+    return STREAM ? __builtin_nontemporal_load(p) : *p;
 }
-__device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
+template <bool STREAM> __device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {
-    if (TBV_NT_OUT) __builtin_nontemporal_store(v, p); else *p = v;
+    __builtin_nontemporal_store(v, p);
 }
-__device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
+template <bool STREAM> __device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {
-    if (TBV_NT_BOUNCE) __builtin_nontemporal_store(v, p); else *p = v;
+    if (STREAM) __builtin_nontemporal_store(v, p); else *p = v;
 }
 
 static constexpr int kThreads = 256;        // 4 wavefronts of 64
@@ -122,9 +120,10 @@ __device__ __forceinline__ void store_sys(unsigned long long* p, unsigned long l
     __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// Every thread of the block calls this after its last store.  When the last
-// block of the grid gets here, all stores of the whole grid are visible system
-// wide and `word` is set to `seq`.
+// Every thread of the block calls this after its last store.  `bid` of `nblk` is the
+// block's index among the blocks being counted (the whole grid, or one part of a merged
+// launch).  When the last of them gets here, all their stores are visible system wide
+// and `word` is set to `seq`.
 //
 // Blocks are counted in two levels so that no single address takes one atomic
 // per block (same-address atomics retire one at a time): groups of kGroup blocks
@@ -143,7 +142,7 @@ static constexpr unsigned kGroup = 32;
 static constexpr unsigned kCtrLine = 16;       // words per counter line (64 bytes)
 
 __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
-                                              unsigned int* ctr, unsigned int nblk, int mode)
+                                              unsigned int* ctr, unsigned int bid, unsigned int nblk, int mode)
 {
     if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -152,7 +151,7 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
         if (mode == 1) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
         bool last = true;
         if (nblk > 1) {
-            const unsigned g = blockIdx.x / kGroup, ngroups = (nblk + kGroup - 1) / kGroup;
+            const unsigned g = bid / kGroup, ngroups = (nblk + kGroup - 1) / kGroup;
             const unsigned pop = min(kGroup, nblk - g * kGroup);
             unsigned int* gc = ctr + kCtrLine * (1 + g);
             last = false;
@@ -223,49 +222,46 @@ struct StepArgs {
     // common
     const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp; int sigmode;
     unsigned long long* pre_word; unsigned long long pre_seq;
+    unsigned pack_blocks;       // merged launch: blocks [0, pack_blocks) pack, the rest sum
 };
 
-template <int DT, int U, bool PACK, bool SUM>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
+// Block `bid` of `nblk` does its share of the payload; block 0 also does the bytes past the last whole vector.
+template <int DT, int U, bool PACK, bool SUM, bool STREAM>
+__device__ __forceinline__ void step_body(const StepArgs& g, unsigned bid, unsigned nblk)
 {
     const unsigned tid = threadIdx.x, nthr = blockDim.x;
-    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);     // deferred signal of the kernel before
-    if (PACK && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
-    if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
-
     const size_t nvec = g.nbytes >> 4;
     const size_t tile = (size_t)nthr * U;
-    for (size_t base = (size_t)blockIdx.x * tile; base < nvec; base += (size_t)gridDim.x * tile) {
+    for (size_t base = (size_t)bid * tile; base < nvec; base += (size_t)nblk * tile) {
         u32x4 x[U], y[U];
         if (base + tile <= nvec) {                       // whole tile: no per-vector bounds checks
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
-                x[u] = ld_a(g.a + i);
-                if (SUM) y[u] = ld_b(g.b + i);
+                x[u] = ld_a<STREAM, PACK && SUM>(g.a + i);
+                if (SUM) y[u] = ld_b<STREAM>(g.b + i);
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
-                if (PACK) st_bounce(g.bounce + i, x[u]);
-                if (SUM) st_out(g.out + i, add_vec<DT>(x[u], y[u]));
+                if (PACK) st_bounce<STREAM>(g.bounce + i, x[u]);
+                if (SUM) st_out<STREAM>(g.out + i, add_vec<DT>(x[u], y[u]));
             }
         } else {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const size_t i = base + (size_t)u * nthr + tid;
                 if (i < nvec) {
-                    x[u] = ld_a(g.a + i);
-                    if (SUM) y[u] = ld_b(g.b + i);
-                    if (PACK) st_bounce(g.bounce + i, x[u]);
-                    if (SUM) st_out(g.out + i, add_vec<DT>(x[u], y[u]));
+                    x[u] = ld_a<STREAM, PACK && SUM>(g.a + i);
+                    if (SUM) y[u] = ld_b<STREAM>(g.b + i);
+                    if (PACK) st_bounce<STREAM>(g.bounce + i, x[u]);
+                    if (SUM) st_out<STREAM>(g.out + i, add_vec<DT>(x[u], y[u]));
                 }
             }
         }
     }
-    // bytes past the last whole vector
     const unsigned tail = (unsigned)(g.nbytes & 15);
-    if (tail && blockIdx.x == 0) {
+    if (tail && bid == 0) {
         const size_t off = nvec << 4;
         if (PACK && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
         if (SUM) {
@@ -279,12 +275,49 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
             }
         }
     }
+}
+
+template <int DT, int U, bool PACK, bool SUM, bool STREAM>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
+{
+    const unsigned tid = threadIdx.x;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);     // deferred signal of the kernel before
+    if (PACK && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    if (SUM && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    step_body<DT, U, PACK, SUM, STREAM>(g, blockIdx.x, gridDim.x);
     if (PACK) {
         if (g.tagp && blockIdx.x == 0 && tid == 0) *g.tagp = g.seq;
-        if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
+        if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
     }
-    if (SUM && g.done) {
-        grid_complete(g.done, g.seq, g.done_arrive, gridDim.x, 1);
+    if (SUM && g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+}
+
+// ---------------------------------------------------------------- the merged launch
+//
+// Pack and sum of one call in ONE launch, as two sets of blocks: blocks [0, P) copy the
+// local tensor into the bounce slot and count themselves complete (the pack's completion
+// word is raised as soon as those P blocks are done, not at the end of the kernel), the
+// remaining blocks sum.  Every kernel in a stream costs about 2.4 us of launch-to-launch
+// time on this GPU whatever it does, so the 16 MiB step drops from 15.2-16.0 us (two
+// launches) to 12.9-13.6 us on cache-cold buffers and from 10.9 to 9.6 us on resident
+// ones.  The sum blocks read the local tensor themselves (the step still moves 5 bytes
+// per payload byte, of which the second read of the local tensor usually hits the
+// Infinity Cache).  Only legal when the received payload is already in place: there is
+// no gate in this kernel.
+template <int DT, int UP, int US, bool STREAM>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_merged(StepArgs g)
+{
+    const unsigned tid = threadIdx.x, P = g.pack_blocks;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    if (blockIdx.x < P) {
+        step_body<DT, UP, true, false, STREAM>(g, blockIdx.x, P);
+        if (g.tagp && blockIdx.x == 0 && tid == 0) *g.tagp = g.seq;
+        if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, P, g.sigmode);
+    } else {
+        const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
+        step_body<DT, US, false, true, STREAM>(g, bid, S);
+        if (g.done) grid_complete(g.done, g.seq, g.done_arrive, bid, S, 1);
     }
 }
 
@@ -309,11 +342,11 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_small_call(StepArgs g)
     const unsigned tail = (unsigned)(g.nbytes & 15);
     const size_t off = nvec << 4;
     u32x4 x = {0, 0, 0, 0};
-    if (mine) { x = ld_a(g.a + i); st_bounce(g.bounce + i, x); }
+    if (mine) { x = ld_a<false, true>(g.a + i); st_bounce<false>(g.bounce + i, x); }
     if (tail && blockIdx.x == 0 && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
-    grid_complete(g.cflag, g.seq, g.pack_arrive, gridDim.x, g.sigmode);
+    grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
     if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
-    if (mine) st_out(g.out + i, add_vec<DT>(x, ld_b(g.b + i)));
+    if (mine) st_out<false>(g.out + i, add_vec<DT>(x, ld_b<false>(g.b + i)));
     if (tail && blockIdx.x == 0) {
         typedef typename Elem<DT>::T T;
         const unsigned ne = tail / sizeof(T);
@@ -324,7 +357,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_small_call(StepArgs g)
             po[tid] = Elem<DT>::add(pa[tid], pb[tid]);
         }
     }
-    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, gridDim.x, 1);
+    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
 
 // Fallback bodies for caller pointers that are not 16-byte aligned: element (sum)
@@ -341,7 +374,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_narrow(PackArgs a)
     if (blockIdx.x == 0 && threadIdx.x < tail)
         ((unsigned char*)a.dst)[n * sizeof(W) + threadIdx.x] = ((const unsigned char*)a.src)[n * sizeof(W) + threadIdx.x];
     if (a.tagp && blockIdx.x == 0 && threadIdx.x == 0) *a.tagp = a.seq;
-    if (a.cflag) grid_complete(a.cflag, a.seq, a.arrive, gridDim.x, a.sigmode);
+    if (a.cflag) grid_complete(a.cflag, a.seq, a.arrive, blockIdx.x, gridDim.x, a.sigmode);
 }
 
 template <int DT>
@@ -354,7 +387,7 @@ __global__ __launch_bounds__(kThreads) void k_sum_narrow(SumArgs a)
     const T* x = (const T*)a.a; const T* y = (const T*)a.b; T* o = (T*)a.out;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
         o[i] = Elem<DT>::add(x[i], y[i]);
-    if (a.done) grid_complete(a.done, a.seq, a.done_arrive, gridDim.x, 1);
+    if (a.done) grid_complete(a.done, a.seq, a.done_arrive, blockIdx.x, gridDim.x, 1);
 }
 
 // ---------------------------------------------------------------- diagnostics
@@ -386,14 +419,21 @@ __global__ void k_fill_u32(unsigned int* p, unsigned int v, size_t n)
 }
 
 // ---------------------------------------------------------------- launch geometry
+//
+// Measured on MI355X with the 16 MiB step (two launches, microseconds per step, cache-cold
+// / cache-resident buffers): resident hints, one vector per lane, 1024 blocks 15.98 / 10.86;
+// streaming hints, four vectors per lane, 1024 blocks 14.18 / 11.18; more blocks (2048,
+// 4096) or 512/1024-lane blocks change nothing; fewer (256, 512) lose 10-40 %.
 
-static int g_unroll = 1;        // vectors per lane per iteration for the large path
+static int g_unroll = 0;        // vectors per lane per iteration for the large path; 0 = the profile's choice
 static int g_grid_cap = 1024;
+static bool g_grid_cap_given = false;   // a cap from the environment applies to every launch shape
 static int g_block = kThreads;
+static bool g_stream = false;   // streaming profile (see the cache hints above)
 
 struct Geom { int grid, block, unroll; };
 
-static Geom geom_for(size_t nbytes, bool writeback = false)
+static Geom geom_for(size_t nbytes, bool writeback = false, bool merged = false)
 {
     size_t nvec = nbytes >> 4;
     Geom g;
@@ -405,10 +445,18 @@ static Geom geom_for(size_t nbytes, bool writeback = false)
         return g;
     }
     g.block = g_block;
-    g.unroll = (nvec >= (size_t)kThreads * 16) ? g_unroll : 1;
+    int cap = g_grid_cap;
+    if (g_unroll) g.unroll = (nvec >= (size_t)kThreads * 16) ? g_unroll : 1;
+    else if (merged) {
+        // the halves of a merged launch run side by side and do best when every block makes a single pass of two
+        // vectors per lane (16 MiB, cold / resident: 12.75 / 9.55 us against 13.05 / 10.2 with 1024 blocks of one)
+        g.unroll = nvec >= (size_t)2 * g_block * 1024 ? 2 : 1;
+        if (!g_grid_cap_given) cap = 2048;
+    }
+    // the streaming profile keeps four loads per lane in flight, as long as that still leaves a block for every grid position
+    else g.unroll = (g_stream && nvec >= (size_t)4 * g_block * g_grid_cap) ? 4 : 1;
     // an L2 write-back per block is dear and they run one after another: use one fat block per CU
-    const int cap = writeback ? 256 : g_grid_cap;
-    if (writeback) g.unroll = 8;
+    if (writeback) { cap = 256; g.unroll = 8; }
     size_t tile = (size_t)g.block * g.unroll;
     size_t tiles = (nvec + tile - 1) / tile;
     g.grid = (int)(tiles < (size_t)cap ? tiles : (size_t)cap);
@@ -419,13 +467,15 @@ static Geom geom_for(size_t nbytes, bool writeback = false)
 int pack_grid(size_t nbytes) { return geom_for(nbytes).grid; }
 int sum_grid(size_t nbytes, int) { return geom_for(nbytes).grid; }
 
-void set_tuning(int unroll, int grid_cap, int block)
+void set_tuning(int unroll, int grid_cap, int block, int streaming)
 {
-    if (block == 256 || block == 512 || block == 1024) g_block = block;
-    if (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) g_unroll = unroll;
+    g_block = (block == 512 || block == 1024) ? block : kThreads;
+    g_unroll = (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) ? unroll : 0;
     // the completion counters have one line per group of kGroup blocks: keep the grid within them
     const int most = (int)(kGroup * (kCounterWords / kCtrLine - 1));
-    if (grid_cap >= 1) g_grid_cap = grid_cap < most ? grid_cap : most;
+    g_grid_cap = grid_cap >= 1 ? (grid_cap < most ? grid_cap : most) : 1024;
+    g_grid_cap_given = grid_cap >= 1;
+    g_stream = streaming != 0;
 }
 
 static inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
@@ -440,25 +490,34 @@ static hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st
     return hipGetLastError();
 }
 
-template <int DT, bool PACK, bool SUM>
+template <int DT, bool PACK, bool SUM, bool STREAM>
 static hipError_t launch_step_u(const StepArgs& s, const Geom& g, hipStream_t st, const Timing* t)
 {
     switch (g.unroll) {
-        case 1: return launch1(k_step<DT, 1, PACK, SUM>, g.grid, g.block, st, t, s);
-        case 2: return launch1(k_step<DT, 2, PACK, SUM>, g.grid, g.block, st, t, s);
-        case 8: return launch1(k_step<DT, 8, PACK, SUM>, g.grid, g.block, st, t, s);
-        default: return launch1(k_step<DT, 4, PACK, SUM>, g.grid, g.block, st, t, s);
+        case 1: return launch1(k_step<DT, 1, PACK, SUM, STREAM>, g.grid, g.block, st, t, s);
+        case 2: return launch1(k_step<DT, 2, PACK, SUM, STREAM>, g.grid, g.block, st, t, s);
+        case 8: return launch1(k_step<DT, 8, PACK, SUM, STREAM>, g.grid, g.block, st, t, s);
+        default: return launch1(k_step<DT, 4, PACK, SUM, STREAM>, g.grid, g.block, st, t, s);
     }
 }
 
 template <bool PACK, bool SUM>
 static hipError_t launch_step(int dtype, const StepArgs& s, const Geom& g, hipStream_t st, const Timing* t)
 {
-    if (!SUM) return launch_step_u<0, PACK, SUM>(s, g, st, t);      // the copy does not depend on the element type
+    if (g_stream) {
+        if (!SUM) return launch_step_u<0, PACK, SUM, true>(s, g, st, t);      // the copy does not depend on the element type
+        switch (dtype) {
+            case 0: return launch_step_u<0, PACK, SUM, true>(s, g, st, t);
+            case 1: return launch_step_u<1, PACK, SUM, true>(s, g, st, t);
+            case 2: return launch_step_u<2, PACK, SUM, true>(s, g, st, t);
+        }
+        return hipErrorInvalidValue;
+    }
+    if (!SUM) return launch_step_u<0, PACK, SUM, false>(s, g, st, t);
     switch (dtype) {
-        case 0: return launch_step_u<0, PACK, SUM>(s, g, st, t);
-        case 1: return launch_step_u<1, PACK, SUM>(s, g, st, t);
-        case 2: return launch_step_u<2, PACK, SUM>(s, g, st, t);
+        case 0: return launch_step_u<0, PACK, SUM, false>(s, g, st, t);
+        case 1: return launch_step_u<1, PACK, SUM, false>(s, g, st, t);
+        case 2: return launch_step_u<2, PACK, SUM, false>(s, g, st, t);
     }
     return hipErrorInvalidValue;
 }
@@ -503,19 +562,56 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
     }
 }
 
-hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+static bool fill_pack_sum(StepArgs& s, const PackArgs& p, const SumArgs& q)
 {
-    if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes)
-        return hipErrorInvalidValue;
-    if (q.done && !q.done_arrive) return hipErrorInvalidValue;
-    if (q.wait_flag) return hipErrorInvalidValue;     // waiting for the peer before sending to it would deadlock two real ranks
-    StepArgs s{};
+    if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes || !p.dst || !q.out || !q.b)
+        return false;
+    if (q.dtype < 0 || q.dtype > 2 || (q.done && !q.done_arrive) || (p.cflag && !p.arrive)) return false;
+    if (q.wait_flag) return false;     // waiting for the peer before sending to it would deadlock two real ranks
     s.bounce = (u32x4*)p.dst; s.cflag = p.cflag; s.pack_arrive = p.arrive; s.tagp = p.tagp;
-    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = nullptr; s.relay = nullptr; s.spin_limit = 0;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.a = (const u32x4*)p.src; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp; s.sigmode = p.sigmode;
     s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
+    return true;
+}
+
+hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+{
+    StepArgs s{};
+    if (!fill_pack_sum(s, p, q)) return hipErrorInvalidValue;
     return launch_step<true, true>(q.dtype, s, geom_for(p.nbytes, p.sigmode != 0), st, t);
+}
+
+template <int DT, bool STREAM>
+static hipError_t launch_merged_u(const StepArgs& s, int grid, int block, int unroll, hipStream_t st, const Timing* t)
+{
+    switch (unroll) {
+        case 2: return launch1(k_merged<DT, 2, 2, STREAM>, grid, block, st, t, s);
+        case 4: return launch1(k_merged<DT, 4, 4, STREAM>, grid, block, st, t, s);
+        default: return launch1(k_merged<DT, 1, 1, STREAM>, grid, block, st, t, s);
+    }
+}
+
+hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+{
+    StepArgs s{};
+    if (!fill_pack_sum(s, p, q) || p.sigmode != 0) return hipErrorInvalidValue;
+    const Geom g = geom_for(p.nbytes, false, true);
+    s.pack_blocks = (unsigned)g.grid;
+    const int grid = 2 * g.grid, u = g.unroll == 8 ? 4 : g.unroll;
+    if (g_stream) {
+        switch (q.dtype) {
+            case 0: return launch_merged_u<0, true>(s, grid, g.block, u, st, t);
+            case 1: return launch_merged_u<1, true>(s, grid, g.block, u, st, t);
+            default: return launch_merged_u<2, true>(s, grid, g.block, u, st, t);
+        }
+    }
+    switch (q.dtype) {
+        case 0: return launch_merged_u<0, false>(s, grid, g.block, u, st, t);
+        case 1: return launch_merged_u<1, false>(s, grid, g.block, u, st, t);
+        default: return launch_merged_u<2, false>(s, grid, g.block, u, st, t);
+    }
 }
 
 int small_call_blocks(size_t nbytes)

@@ -64,6 +64,8 @@ def _bind(so):
     l.tbv_ar_allreduce_chunked.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce_chunked.restype = ci
     l.tbv_emu_run_pack.argtypes = [vp, sz, ci, vp]; l.tbv_emu_run_pack.restype = ci
     l.tbv_emu_run_sum.argtypes = [vp, vp, vp, sz, ci, vp]; l.tbv_emu_run_sum.restype = ci
+    l.tbv_emu_hbm_probe.argtypes = [ci, sz, sz, ci, dp, dp]; l.tbv_emu_hbm_probe.restype = ci
+    l.tbv_emu_launch_floor.argtypes = [ci, dp]; l.tbv_emu_launch_floor.restype = ci
     return l
 
 
@@ -248,6 +250,24 @@ def kernel_times(which):
     m, mn = ctypes.c_double(), ctypes.c_double()
     n = _lib.tbv_emu_kernel_times(which, ctypes.byref(m), ctypes.byref(mn))
     return n, m.value, mn.value
+
+
+def hbm_probe(kind, nbytes, pool_bytes, reps, so=_DEFAULT_SO):
+    """(mean_us, min_us) of a plain streaming kernel: kind 0 read, 1 write, 2 non-temporal copy, 3 plain copy."""
+    l = _lib or load(so)
+    m, mn = ctypes.c_double(), ctypes.c_double()
+    if l.tbv_emu_hbm_probe(kind, nbytes, pool_bytes, reps, ctypes.byref(m), ctypes.byref(mn)) != 0:
+        raise RuntimeError("tbv_emu_hbm_probe failed")
+    return m.value, mn.value
+
+
+def launch_floor(reps=2000, so=_DEFAULT_SO):
+    """Launch-to-launch microseconds of an empty kernel in one stream."""
+    l = _lib or load(so)
+    v = ctypes.c_double()
+    if l.tbv_emu_launch_floor(reps, ctypes.byref(v)) != 0:
+        raise RuntimeError("tbv_emu_launch_floor failed")
+    return v.value
 
 
 def footprints():

@@ -182,6 +182,9 @@ MODES = {
     "nslot32": {"TBV_NSLOT": 32},
     "unroll4": {"TBV_UNROLL": 4, "TBV_GRIDCAP": 200},
     "pin": {"TBV_CPU": 0},
+    "streaming": {"TBV_STREAMING": 1},
+    "streaming_unroll2": {"TBV_STREAMING": 1, "TBV_UNROLL": 2},
+    "merge_off": {"TBV_MERGE": 0},
 }
 
 
@@ -227,8 +230,8 @@ def test_resident_peer_fused_and_unfused(orc):
     a = dev(synth.prefill_activations(100, n // 2), torch.bfloat16)
     b = dev(synth.prefill_activations(101, n // 2), torch.bfloat16)
     want = oracle_sum(orc, a, b)
-    for fuse in (0, 1):
-        with session(rails=2, cap=n, TBV_FUSE=fuse) as tbv:
+    for fuse, merge, streaming in ((0, 1, 0), (1, 1, 0), (0, 0, 0), (0, 1, 1), (1, 1, 1), (0, 0, 1)):
+        with session(rails=2, cap=n, TBV_FUSE=fuse, TBV_MERGE=merge, TBV_STREAMING=streaming) as tbv:
             tbv.peer_resident(b)
             out = torch.empty_like(a)
             for _ in range(9):
@@ -253,6 +256,39 @@ def test_resident_peer_fused_and_unfused(orc):
             assert torch.equal(o2, small + b[:4096]) and torch.equal(o3, small + p3)
             tbv.peer_resident(None)
             assert not tbv.err()
+
+
+@pytest.mark.parametrize("streaming", [0, 1])
+def test_resident_peer_merged_launch_ragged(orc, streaming):
+    """Early peer above the one-kernel size: pack blocks and sum blocks share one launch.  Ragged byte counts,
+    three dtypes, in place and out of place, slots reused; the bounce image is read back too."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so.7")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    cap = 6 << 20
+    with session(rails=2, cap=cap, TBV_NSLOT=3, TBV_STREAMING=streaming, TBV_UNROLL=(2 if streaming else 0)) as tbv:
+        for name in ("bf16", "f16", "f32"):
+            dt = DT[name]
+            esz = 4 if name == "f32" else 2
+            peer = dev(synth.uniform(70, cap // esz), dt)
+            tbv.peer_resident(peer)
+            for k, numel in enumerate(((1 << 20) // esz + 1, (3 << 20) // esz + 7, cap // esz, (2 << 20) // esz + 3, (5 << 20) // esz - 1)):
+                a = dev(synth.uniform(71 + k, numel), dt)
+                want = oracle_sum(orc, a, peer[:numel])
+                out = torch.empty_like(a)
+                say("merged", name, numel, "streaming", streaming)
+                assert tbv.all_reduce(a, out)
+                torch.cuda.synchronize()
+                assert first_diff(out, want) is None, (name, numel)
+                img = torch.empty_like(a)
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), numel * esz, 3) == 0
+                assert np.array_equal(bits_np(img), bits_np(a))
+                c = a.clone()
+                assert tbv.all_reduce(c)                               # in place
+                torch.cuda.synchronize()
+                assert first_diff(c, want) is None, (name, numel, "in place")
+            tbv.peer_resident(None)
+        assert not tbv.err()
 
 
 def test_full_size_properties(orc):
