@@ -180,6 +180,25 @@ int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, int dtype, vo
 int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream);
 int tbv_emu_run_sum(void* out, const void* a, const void* b, size_t nbytes, int dtype, void* stream);
 
+/* One step of the data path with no allocation anywhere.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It needs no tbv_ar_init.
+ *   bounce <- local (nbytes), then *pack_word = seq once every byte of it is visible;
+ *   out <- local + received in `dtype`, then *done_word = seq.
+ * All five buffers are the caller's, 16-byte aligned device memory; out may alias local.
+ * bounce_uncached != 0 says that `bounce` is uncached (fine-grained) memory.  pack_word
+ * and done_word are host-visible or device words, either may be NULL.  The kernels count
+ * their blocks in a 16 KiB device array built into the library (one copy per GPU, held
+ * until the process ends), so no hipMalloc, hipFree or other allocating call is made.
+ * Calls that overlap in time on one GPU share that array and race: issue them on one
+ * stream, or otherwise one after the other.  Returns 0; -2 when nbytes exceeds
+ * TBV_NOALLOC_MAX_BYTES; -1 for bad arguments or a launch failure ("[tbvcoll] ..." on
+ * stderr says which). */
+#define TBV_NOALLOC_MAX_BYTES ((size_t)1 << 30)
+int tbv_step_noalloc(void* out, const void* local, const void* received, void* bounce, int bounce_uncached,
+                     size_t nbytes, int dtype, unsigned long long* pack_word, unsigned long long* done_word,
+                     unsigned long long seq, void* stream);
+
 /* What plain streaming kernels reach on this GPU, as measured denominators beside the
  * published HBM peak (no counterpart in the reference).  tbv_emu_hbm_probe streams
  * `bytes` per launch (kind 0 read, 1 write, 2 copy with non-temporal accesses, 3 plain

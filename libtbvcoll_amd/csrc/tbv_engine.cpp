@@ -823,6 +823,7 @@ static int init_impl(int rank, const char* devs, size_t cap)
       if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, G.device) == hipSuccess && khz > 0) G.tick_hz = khz * 1e3;
       (void)hipGetLastError(); }
 
+    if (!tbv::noalloc_bind_device()) FAIL("built-in counter array not addressable on device %d", G.device);
     const size_t span = G.stride * (size_t)G.nslot;
     if (!alloc_slab(&G.sendbase, span, (G.uncached & 1) != 0, g_uc_send)) FAIL("send bounce allocation failed (%zu B)", span);
     if (!alloc_slab(&G.recvbase, span, (G.uncached & 2) != 0, g_uc_recv)) FAIL("receive bounce allocation failed (%zu B)", span);

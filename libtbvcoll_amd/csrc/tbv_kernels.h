@@ -83,4 +83,7 @@ hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, 
 hipError_t launch_mark(unsigned long long* fp, int i, unsigned long long seq, hipStream_t st);
 hipError_t launch_fill_u32(unsigned int* p, unsigned int v, size_t n, hipStream_t st);
 
+// Looks up this device's copy of the built-in counter array of tbv_step_noalloc (once per device).
+bool noalloc_bind_device();
+
 }  // namespace tbv

@@ -64,6 +64,7 @@ def _bind(so):
     l.tbv_ar_allreduce_chunked.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce_chunked.restype = ci
     l.tbv_emu_run_pack.argtypes = [vp, sz, ci, vp]; l.tbv_emu_run_pack.restype = ci
     l.tbv_emu_run_sum.argtypes = [vp, vp, vp, sz, ci, vp]; l.tbv_emu_run_sum.restype = ci
+    l.tbv_step_noalloc.argtypes = [vp, vp, vp, vp, ci, sz, ci, vp, vp, ctypes.c_ulonglong, vp]; l.tbv_step_noalloc.restype = ci
     l.tbv_emu_hbm_probe.argtypes = [ci, sz, sz, ci, dp, dp]; l.tbv_emu_hbm_probe.restype = ci
     l.tbv_emu_launch_floor.argtypes = [ci, dp]; l.tbv_emu_launch_floor.restype = ci
     return l
