@@ -119,8 +119,8 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     tbv.stats4()
     for _ in range(min(nslot - 1, 12)):
         step()
+    torch.cuda.synchronize()           # the averages are per completed transfer: let all of them complete
     enq = tbv.stats4()[3]
-    torch.cuda.synchronize()
     want = a + b
     ok = all(bool(torch.equal(o, want)) for o in outs)    # the timed path computed the sum, bit for bit
     tbv.stats4()

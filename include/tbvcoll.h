@@ -116,6 +116,12 @@ int tbv_emu_arrival_script(const int* rails, size_t n);
  * seq == 0 clears. */
 int tbv_emu_withhold(unsigned long long seq, int rail);
 
+/* Test hook: while `hold` is non-zero, rail `rail` deposits nothing; each held transfer is
+ * bounded by the watchdog.  Setting a hold needs idle rails; lifting it may be done at
+ * any time and from any thread (the one emulated-peer call that may be made while
+ * another thread is inside tbv_ar_allreduce). */
+int tbv_emu_hold_rail(int rail, int hold);
+
 /* Sequence number of the last call issued (0 before the first). */
 unsigned long long tbv_emu_seq(void);
 

@@ -1,19 +1,22 @@
 """tbvcoll -- ctypes binding of libtbvcoll.so (MI355X build).
 
-Same module surface as the reference binding (step4/tbvcoll.py:14-111): `init`,
-`all_reduce`, `is_async`, `err`, `rails`, `hist`, `raw_fn`, `cap`, `stats`,
-`stats3`, `stats4`, `stats5`, with the same guards and return conventions, so a
-caller written against the reference (an exact/stress driver, a vLLM
-`GroupCoordinator.all_reduce` intercept) runs unchanged.
+The module keeps the surface of the reference binding (step4/tbvcoll.py:14-111): `init`,
+`all_reduce`, `is_async`, `err`, `rails`, `hist`, `raw_fn`, `cap`, `stats`, `stats3`,
+`stats4`, `stats5`, with the same guards and return conventions, so a caller written
+against the reference (a vLLM `GroupCoordinator.all_reduce` intercept, code that uses the
+C function through `raw_fn`) binds without changes.  On one GPU the peer is emulated: a
+two-rank exact/stress driver additionally has to hand over the peer's payload with
+`stage_peer` before each call (without one the peer echoes this rank's own payload).
 
     import tbvcoll
     tbvcoll.init(rank, "rail0,rail1", "", cap_bytes=8 << 20)
+    tbvcoll.stage_peer(peer_tensor)    # this build only: what the other rank would have sent
     tbvcoll.all_reduce(t)              # in-place SUM; False -> caller falls back
 
-Additions (no counterpart in the reference) drive the emulated peer that
-replaces the wire: `stage_peer`, `stage_peer_repeat`, `peer_resident`,
-`arrival_script`, `withhold`, `latency_probe`, `latencies`, `arrival_log`,
-`all_reduce_chunked`, `shutdown`, `lib`.
+Additions (no counterpart in the reference): the emulated peer (`stage_peer`,
+`stage_peer_repeat`, `peer_resident`, `arrival_script`, `hold_rail`, `withhold`,
+`arrival_log`), measurement (`latency_probe`, `latencies`, `kernel_timing`, `kernel_times`,
+`hbm_probe`, `launch_floor`), `all_reduce_chunked`, `shutdown`, `lib`.
 
 There is no CPU fallback: if the shared library is missing, `init` raises.
 """
@@ -27,46 +30,39 @@ _lib = None
 _cap = 0
 _DEFAULT_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtbvcoll.so")
 
+_VP, _SZ, _I, _U64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_ulonglong
+_PD, _PU, _PI, _PSZ = (ctypes.POINTER(t) for t in (ctypes.c_double, ctypes.c_ulonglong, ctypes.c_int, ctypes.c_size_t))
+
+# symbol -> (restype, argtypes): everything include/tbvcoll.h declares
+_SIGNATURES = {
+    "tbv_ar_init": (_I, [_I, ctypes.c_char_p, ctypes.c_char_p, _I, _SZ]),
+    "tbv_ar_allreduce": (_I, [_VP, _VP, _SZ, _I, _VP]),
+    "tbv_ar_stats": (None, [_PD, _PU]),
+    "tbv_ar_stats4": (None, [_PD] * 4 + [_PU]),
+    "tbv_ar_stats5": (None, [_PD] * 5 + [_PU]),
+    "tbv_ar_cap": (_I, []), "tbv_ar_async": (_I, []), "tbv_ar_err": (_I, []),
+    "tbv_ar_rails": (None, []), "tbv_ar_hist": (None, []), "tbv_ar_fini": (None, []),
+    "tbv_emu_shutdown": (None, []),
+    "tbv_emu_stage_peer": (_I, [_VP, _SZ]), "tbv_emu_stage_peer_repeat": (_I, [_VP, _SZ]), "tbv_emu_peer_resident": (_I, [_VP, _SZ]),
+    "tbv_emu_arrival_script": (_I, [_PI, _SZ]), "tbv_emu_withhold": (_I, [_U64, _I]), "tbv_emu_hold_rail": (_I, [_I, _I]),
+    "tbv_emu_seq": (_U64, []), "tbv_emu_plan": (_I, [_SZ, _PSZ, _PSZ]), "tbv_emu_configure": (_I, [ctypes.c_char_p, _SZ]),
+    "tbv_emu_nslot": (_I, []), "tbv_emu_stride": (_SZ, []), "tbv_emu_send_slot": (_VP, [_I]), "tbv_emu_recv_slot": (_VP, [_I]),
+    "tbv_emu_arrival_log": (_SZ, [_PU, _PI, _SZ]),
+    "tbv_emu_latency_probe": (_I, [_I]), "tbv_emu_latencies": (_SZ, [_PD, _SZ]),
+    "tbv_emu_kernel_timing": (_I, [_I]), "tbv_emu_kernel_times": (_SZ, [_I, _PD, _PD]),
+    "tbv_emu_footprints": (None, [_PU]), "tbv_emu_tag_counts": (None, [_PU, _PU, _PU]),
+    "tbv_ar_allreduce_chunked": (_I, [_VP, _VP, _SZ, _I, _VP]),
+    "tbv_emu_run_pack": (_I, [_VP, _SZ, _I, _VP]), "tbv_emu_run_sum": (_I, [_VP, _VP, _VP, _SZ, _I, _VP]),
+    "tbv_step_noalloc": (_I, [_VP, _VP, _VP, _VP, _I, _SZ, _I, _VP, _VP, _U64, _VP]),
+    "tbv_emu_hbm_probe": (_I, [_I, _SZ, _SZ, _I, _PD, _PD]), "tbv_emu_launch_floor": (_I, [_I, _PD]),
+}
+
 
 def _bind(so):
     l = ctypes.CDLL(so)
-    vp, sz, ci, dp, up = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), \
-        ctypes.POINTER(ctypes.c_ulonglong)
-    l.tbv_ar_init.argtypes = [ci, ctypes.c_char_p, ctypes.c_char_p, ci, sz]; l.tbv_ar_init.restype = ci
-    l.tbv_ar_allreduce.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce.restype = ci
-    l.tbv_ar_stats.argtypes = [dp, up]; l.tbv_ar_stats.restype = None
-    l.tbv_ar_stats4.argtypes = [dp] * 4 + [up]; l.tbv_ar_stats4.restype = None
-    l.tbv_ar_stats5.argtypes = [dp] * 5 + [up]; l.tbv_ar_stats5.restype = None
-    for name in ("tbv_ar_async", "tbv_ar_err", "tbv_ar_cap"):
-        getattr(l, name).argtypes = []; getattr(l, name).restype = ci
-    for name in ("tbv_ar_rails", "tbv_ar_hist", "tbv_ar_fini", "tbv_emu_shutdown"):
-        getattr(l, name).argtypes = []; getattr(l, name).restype = None
-    # emulated peer
-    l.tbv_emu_stage_peer.argtypes = [vp, sz]; l.tbv_emu_stage_peer.restype = ci
-    l.tbv_emu_stage_peer_repeat.argtypes = [vp, sz]; l.tbv_emu_stage_peer_repeat.restype = ci
-    l.tbv_emu_peer_resident.argtypes = [vp, sz]; l.tbv_emu_peer_resident.restype = ci
-    l.tbv_emu_arrival_script.argtypes = [ctypes.POINTER(ci), sz]; l.tbv_emu_arrival_script.restype = ci
-    l.tbv_emu_withhold.argtypes = [ctypes.c_ulonglong, ci]; l.tbv_emu_withhold.restype = ci
-    l.tbv_emu_seq.argtypes = []; l.tbv_emu_seq.restype = ctypes.c_ulonglong
-    l.tbv_emu_plan.argtypes = [sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]; l.tbv_emu_plan.restype = ci
-    l.tbv_emu_configure.argtypes = [ctypes.c_char_p, sz]; l.tbv_emu_configure.restype = ci
-    l.tbv_emu_nslot.argtypes = []; l.tbv_emu_nslot.restype = ci
-    l.tbv_emu_stride.argtypes = []; l.tbv_emu_stride.restype = sz
-    l.tbv_emu_send_slot.argtypes = [ci]; l.tbv_emu_send_slot.restype = vp
-    l.tbv_emu_recv_slot.argtypes = [ci]; l.tbv_emu_recv_slot.restype = vp
-    l.tbv_emu_arrival_log.argtypes = [up, ctypes.POINTER(ci), sz]; l.tbv_emu_arrival_log.restype = sz
-    l.tbv_emu_latency_probe.argtypes = [ci]; l.tbv_emu_latency_probe.restype = ci
-    l.tbv_emu_latencies.argtypes = [dp, sz]; l.tbv_emu_latencies.restype = sz
-    l.tbv_emu_kernel_timing.argtypes = [ci]; l.tbv_emu_kernel_timing.restype = ci
-    l.tbv_emu_kernel_times.argtypes = [ci, dp, dp]; l.tbv_emu_kernel_times.restype = sz
-    l.tbv_emu_footprints.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]; l.tbv_emu_footprints.restype = None
-    l.tbv_emu_tag_counts.argtypes = [up, up, up]; l.tbv_emu_tag_counts.restype = None
-    l.tbv_ar_allreduce_chunked.argtypes = [vp, vp, sz, ci, vp]; l.tbv_ar_allreduce_chunked.restype = ci
-    l.tbv_emu_run_pack.argtypes = [vp, sz, ci, vp]; l.tbv_emu_run_pack.restype = ci
-    l.tbv_emu_run_sum.argtypes = [vp, vp, vp, sz, ci, vp]; l.tbv_emu_run_sum.restype = ci
-    l.tbv_step_noalloc.argtypes = [vp, vp, vp, vp, ci, sz, ci, vp, vp, ctypes.c_ulonglong, vp]; l.tbv_step_noalloc.restype = ci
-    l.tbv_emu_hbm_probe.argtypes = [ci, sz, sz, ci, dp, dp]; l.tbv_emu_hbm_probe.restype = ci
-    l.tbv_emu_launch_floor.argtypes = [ci, dp]; l.tbv_emu_launch_floor.restype = ci
+    for name, (res, args) in _SIGNATURES.items():
+        f = getattr(l, name)                   # AttributeError names the missing symbol
+        f.restype, f.argtypes = res, args
     return l
 
 
@@ -89,26 +85,36 @@ def init(rank, devs, peer_ip, port=18995, cap_bytes=8 << 20, so=_DEFAULT_SO):
     _lib, _cap = l, l.tbv_ar_cap()
 
 
+def _call_args(t, out):
+    """(in_ptr, out_ptr, nbytes, dtype code) of a tensor pair the library can take, or None: not initialised,
+    not on the GPU, not contiguous, mismatched output, unsupported dtype (the guards of step4/tbvcoll.py:38-47)."""
+    if _lib is None or not t.is_cuda or not t.is_contiguous():
+        return None
+    if out is not None and (not out.is_contiguous() or out.dtype is not t.dtype or out.numel() != t.numel()):
+        return None
+    code = _DT.get(t.dtype)
+    if code is None:
+        return None
+    return _VP(t.data_ptr()), (_VP(out.data_ptr()) if out is not None else None), t.numel() * t.element_size(), code
+
+
+def _stream():
+    # read on every call: a cached handle goes stale when the caller switches streams
+    return _VP(torch.cuda.current_stream().cuda_stream)
+
+
 def all_reduce(t: torch.Tensor, out: torch.Tensor = None) -> bool:
     """SUM with the peer.  out=None means in place.  False means "not handled
     here, use your own collective" (step4/tbvcoll.py:35-58)."""
-    if _lib is None or not t.is_cuda or not t.is_contiguous():
+    a = _call_args(t, out)
+    if a is None:
         return False
-    if out is not None and (not out.is_contiguous() or out.dtype is not t.dtype or out.numel() != t.numel()):
-        return False
-    dt = _DT.get(t.dtype)
-    if dt is None:
-        return False
-    nb = t.numel() * t.element_size()
+    pin, pout, nb, code = a
     if nb == 0:
         return True
     if nb > _cap:
         return False
-    # the current stream is read on every call: a cached handle goes stale when the caller switches streams
-    st = torch.cuda.current_stream().cuda_stream
-    rc = _lib.tbv_ar_allreduce(ctypes.c_void_p(t.data_ptr()),
-                               ctypes.c_void_p(out.data_ptr()) if out is not None else None,
-                               nb, dt, ctypes.c_void_p(st))
+    rc = _lib.tbv_ar_allreduce(pin, pout, nb, code, _stream())
     if rc == -2:
         return False
     if rc != 0:
@@ -144,32 +150,31 @@ def cap():
     return _cap
 
 
+def _read_stats(fn, ndoubles):
+    vals = [ctypes.c_double() for _ in range(ndoubles)]
+    n = ctypes.c_ulonglong()
+    fn(*[ctypes.byref(v) for v in vals], ctypes.byref(n))
+    return tuple(v.value for v in vals) + (n.value,)
+
+
 def stats5():
     """(pre, xfer, post, enq, drain, count), microseconds per call; reading resets."""
-    a, b, c, d, e = (ctypes.c_double() for _ in range(5))
-    n = ctypes.c_ulonglong()
-    _lib.tbv_ar_stats5(*[ctypes.byref(x) for x in (a, b, c, d, e)], ctypes.byref(n))
-    return a.value, b.value, c.value, d.value, e.value, n.value
+    return _read_stats(_lib.tbv_ar_stats5, 5)
 
 
 def stats4():
     """(pre_us, xfer_us, post_us, enq_us, count)."""
-    a, b, c, d = (ctypes.c_double() for _ in range(4))
-    n = ctypes.c_ulonglong()
-    _lib.tbv_ar_stats4(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c), ctypes.byref(d), ctypes.byref(n))
-    return a.value, b.value, c.value, d.value, n.value
+    return _read_stats(_lib.tbv_ar_stats4, 4)
 
 
 def stats3():
-    pre, xf, post, enq, n = stats4()
+    pre, xf, post, _, n = stats4()
     return pre, xf, post, n
 
 
 def stats():
     """(mean transfer us, calls); reading resets."""
-    a, c = ctypes.c_double(), ctypes.c_ulonglong()
-    _lib.tbv_ar_stats(ctypes.byref(a), ctypes.byref(c))
-    return a.value, c.value
+    return _read_stats(_lib.tbv_ar_stats, 1)
 
 
 # ------------------------------------------------------------------ emulated peer (additive)
@@ -183,13 +188,16 @@ def _nbytes(t):
     return t.numel() * t.element_size()
 
 
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed rc={rc}")
+
+
 def stage_peer(t: torch.Tensor):
     """Queue `t` as the peer's payload of the next call that has none.  Keep `t`
     alive until that call's result is complete."""
     assert t.is_contiguous()
-    rc = _lib.tbv_emu_stage_peer(ctypes.c_void_p(t.data_ptr()), _nbytes(t))
-    if rc != 0:
-        raise RuntimeError(f"tbv_emu_stage_peer failed rc={rc}")
+    _check(_lib.tbv_emu_stage_peer(_VP(t.data_ptr()), _nbytes(t)), "tbv_emu_stage_peer")
 
 
 def stage_peer_repeat(t):
@@ -197,26 +205,25 @@ def stage_peer_repeat(t):
         _lib.tbv_emu_stage_peer_repeat(None, 0)
     else:
         assert t.is_contiguous()
-        _lib.tbv_emu_stage_peer_repeat(ctypes.c_void_p(t.data_ptr()), _nbytes(t))
+        _lib.tbv_emu_stage_peer_repeat(_VP(t.data_ptr()), _nbytes(t))
 
 
 def peer_resident(t):
-    rc = _lib.tbv_emu_peer_resident(None, 0) if t is None else \
-        _lib.tbv_emu_peer_resident(ctypes.c_void_p(t.data_ptr()), _nbytes(t))
-    if rc != 0:
-        raise RuntimeError(f"tbv_emu_peer_resident failed rc={rc}")
+    _check(_lib.tbv_emu_peer_resident(None, 0) if t is None else _lib.tbv_emu_peer_resident(_VP(t.data_ptr()), _nbytes(t)),
+           "tbv_emu_peer_resident")
 
 
 def arrival_script(rails_list):
     n = len(rails_list)
-    arr = (ctypes.c_int * max(n, 1))(*rails_list)
-    rc = _lib.tbv_emu_arrival_script(arr, n)
-    if rc != 0:
-        raise RuntimeError(f"tbv_emu_arrival_script failed rc={rc}")
+    _check(_lib.tbv_emu_arrival_script((ctypes.c_int * max(n, 1))(*rails_list), n), "tbv_emu_arrival_script")
 
 
 def withhold(seq, rail=0):
     _lib.tbv_emu_withhold(seq, rail)
+
+
+def hold_rail(rail, hold=True):
+    _check(_lib.tbv_emu_hold_rail(rail, 1 if hold else 0), "tbv_emu_hold_rail")
 
 
 def seq():
@@ -224,9 +231,7 @@ def seq():
 
 
 def latency_probe(on=True):
-    rc = _lib.tbv_emu_latency_probe(1 if on else 0)
-    if rc != 0:
-        raise RuntimeError("tbv_emu_latency_probe failed")
+    _check(_lib.tbv_emu_latency_probe(1 if on else 0), "tbv_emu_latency_probe")
 
 
 def latencies(max_n=1 << 20):
@@ -257,8 +262,7 @@ def hbm_probe(kind, nbytes, pool_bytes, reps, so=_DEFAULT_SO):
     """(mean_us, min_us) of a plain streaming kernel: kind 0 read, 1 write, 2 non-temporal copy, 3 plain copy."""
     l = _lib or load(so)
     m, mn = ctypes.c_double(), ctypes.c_double()
-    if l.tbv_emu_hbm_probe(kind, nbytes, pool_bytes, reps, ctypes.byref(m), ctypes.byref(mn)) != 0:
-        raise RuntimeError("tbv_emu_hbm_probe failed")
+    _check(l.tbv_emu_hbm_probe(kind, nbytes, pool_bytes, reps, ctypes.byref(m), ctypes.byref(mn)), "tbv_emu_hbm_probe")
     return m.value, mn.value
 
 
@@ -266,8 +270,7 @@ def launch_floor(reps=2000, so=_DEFAULT_SO):
     """Launch-to-launch microseconds of an empty kernel in one stream."""
     l = _lib or load(so)
     v = ctypes.c_double()
-    if l.tbv_emu_launch_floor(reps, ctypes.byref(v)) != 0:
-        raise RuntimeError("tbv_emu_launch_floor failed")
+    _check(l.tbv_emu_launch_floor(reps, ctypes.byref(v)), "tbv_emu_launch_floor")
     return v.value
 
 
@@ -286,19 +289,11 @@ def tag_counts():
 
 def all_reduce_chunked(t: torch.Tensor, out: torch.Tensor = None) -> bool:
     """Pipelined SUM of a tensor of any size as cap-sized chunks."""
-    if _lib is None or not t.is_cuda or not t.is_contiguous():
+    a = _call_args(t, out)
+    if a is None:
         return False
-    if out is not None and (not out.is_contiguous() or out.dtype is not t.dtype or out.numel() != t.numel()):
-        return False
-    dt = _DT.get(t.dtype)
-    if dt is None:
-        return False
-    st = torch.cuda.current_stream().cuda_stream
-    rc = _lib.tbv_ar_allreduce_chunked(ctypes.c_void_p(t.data_ptr()),
-                                       ctypes.c_void_p(out.data_ptr()) if out is not None else None,
-                                       _nbytes(t), dt, ctypes.c_void_p(st))
-    if rc != 0:
-        raise RuntimeError(f"tbv_ar_allreduce_chunked failed rc={rc}")
+    pin, pout, nb, code = a
+    _check(_lib.tbv_ar_allreduce_chunked(pin, pout, nb, code, _stream()), "tbv_ar_allreduce_chunked")
     return True
 
 

@@ -54,6 +54,9 @@ def lib():
         l.orc_ring_model.argtypes = [ctypes.POINTER(sz), sz, ctypes.POINTER(ci), sz, ci, ci, sz, ci,
                                      ctypes.POINTER(u64), ctypes.POINTER(ci), ctypes.POINTER(ci)]
         l.orc_ring_model.restype = ctypes.c_long
+        l.orc_ring_model2.argtypes = [ctypes.POINTER(sz), sz, ctypes.POINTER(ci), sz, ci, ci, sz, ci, ci,
+                                      ctypes.POINTER(u64), ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ctypes.c_long)]
+        l.orc_ring_model2.restype = ctypes.c_long
         l.orc_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci]; l.orc_reduce_copy.restype = ci
         l.orc_time_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci, ci, ci]; l.orc_time_reduce_copy.restype = ctypes.c_double
         _lib = l
@@ -115,6 +118,20 @@ def ring_model(call_nbytes, script, nslot, nrails, rail1max=98304, depth=1):
     rails = (ctypes.c_int * max(n, 1))()
     k = lib().orc_ring_model(calls, n, scr, m, nslot, nrails, rail1max, depth, rel, slots, rails)
     return k, list(rel)[:max(k, 0)], list(slots)[:n], list(rails)[:n]
+
+
+def ring_model2(call_nbytes, script, nslot, nrails, rail1max=98304, depth=1, slot_guard=1):
+    """As ring_model, with the caller optionally holding a call back until its slot's previous user has
+    been released; also returns how many calls were issued into a slot still owned by an unreleased call."""
+    n, m = len(call_nbytes), len(script)
+    calls = (ctypes.c_size_t * max(n, 1))(*call_nbytes)
+    scr = (ctypes.c_int * max(m, 1))(*script)
+    rel = (ctypes.c_uint64 * max(m, 1))()
+    slots = (ctypes.c_int * max(n, 1))()
+    rails = (ctypes.c_int * max(n, 1))()
+    shared = ctypes.c_long(0)
+    k = lib().orc_ring_model2(calls, n, scr, m, nslot, nrails, rail1max, depth, slot_guard, rel, slots, rails, ctypes.byref(shared))
+    return k, list(rel)[:max(k, 0)], list(slots)[:n], list(rails)[:n], shared.value
 
 
 def reduce_copy(dtype, local, peer, nthreads=1):

@@ -203,29 +203,50 @@ int orc_hist_bucket(size_t nbytes) { int b = 0; size_t v = nbytes; while (v >>= 
  */
 typedef struct { uint64_t seq; int slot; int R; } orc_item;
 
-long orc_ring_model(const size_t* call_nbytes, size_t ncalls, const int* script, size_t nscript,
-                    int nslot, int nrails, size_t rail1max, int depth,
-                    uint64_t* released /* [nscript] */, int* slots /* [ncalls] */, int* rails /* [ncalls] */)
+/* slot_guard = 0: the reference's only back-pressure, queue depth per used rail (:441-443).  A
+ * rail's queue holds only the calls that use that rail, so a one-rail call can then be issued
+ * into a slot whose previous, two-rail call still waits for rail 1; the two calls share the
+ * slot's rail counter (rails_done, :105,268-271).  *shared_slot (may be NULL) counts the calls
+ * issued into a slot whose previous user had not been released.
+ * slot_guard = 1: the caller also holds a call back until its slot's previous user (seq - nslot)
+ * has been released; *shared_slot stays 0 and every release names the call whose rails all arrived.
+ * depth <= 0 drops the stream-order limit (a stream cannot pack call s+depth before call s's wait
+ * has passed, which on one stream is a slot guard by itself) and models the host alone: it issues
+ * as long as queue depth (and the guard) allow and otherwise waits for the next arrival.  That is
+ * the situation of a call whose flag does not wait for the stream (peer payload already there). */
+long orc_ring_model2(const size_t* call_nbytes, size_t ncalls, const int* script, size_t nscript,
+                     int nslot, int nrails, size_t rail1max, int depth, int slot_guard,
+                     uint64_t* released /* [nscript] */, int* slots /* [ncalls] */, int* rails /* [ncalls] */,
+                     long* shared_slot)
 {
     enum { MAXR = 4, MAXS = 32 };
     orc_item q[MAXR][MAXS];
     uint64_t head[MAXR] = {0}, tail[MAXR] = {0};
     unsigned rails_done[MAXS] = {0};
     uint64_t gflag[MAXS] = {0};
+    uint64_t slot_released[MAXS] = {0};
     uint64_t seq = 0, done_upto = 0;
     unsigned char rel_seen[64] = {0};          /* released-but-not-yet-retired marks, window <= nslot */
     size_t next_call = 0, k = 0;
+    long shared = 0;
+    const int host_only = depth <= 0;
     if (depth < 1) depth = 1;
     if (depth > nslot) depth = nslot;
     for (;;) {
         /* caller: enqueue while it may run ahead: at most `depth` calls whose release is pending
          * (a single stream cannot pack call s+depth before call s's wait has passed) */
-        while (next_call < ncalls && seq - done_upto < (uint64_t)depth) {
+        while (next_call < ncalls && (host_only || seq - done_upto < (uint64_t)depth)) {
             size_t nb = call_nbytes[next_call];
             int R = orc_rails_for(nb, rail1max, nrails);
-            for (int r = 0; r < R; r++) if (head[r] - tail[r] >= (uint64_t)nslot) return -2;
+            int slot = orc_slot(seq + 1, nslot);
+            int prev_unreleased = seq + 1 > (uint64_t)nslot && slot_released[slot] < seq + 1 - (uint64_t)nslot;
+            int full = 0;
+            if (slot_guard && prev_unreleased) break;             /* wait for an arrival that releases it */
+            for (int r = 0; r < R; r++) if (head[r] - tail[r] >= (uint64_t)nslot) full = 1;
+            if (full && host_only) break;                         /* wait for room in the ring */
+            if (full) return -2;
+            if (prev_unreleased) shared++;
             seq++;
-            int slot = orc_slot(seq, nslot);
             if (slots) slots[next_call] = slot;
             if (rails) rails[next_call] = R;
             for (int r = 0; r < R; r++) { orc_item it = { seq, slot, R }; q[r][head[r] % nslot] = it; head[r]++; }
@@ -238,6 +259,7 @@ long orc_ring_model(const size_t* call_nbytes, size_t ncalls, const int* script,
         uint64_t rel = 0;
         if (++rails_done[it.slot] >= (unsigned)it.R) {
             rails_done[it.slot] = 0; gflag[it.slot] = it.seq; rel = it.seq;
+            if (slot_released[it.slot] < it.seq) slot_released[it.slot] = it.seq;
             /* a 1-rail call may be released before an older 2-rail call; the stream
              * retires waits in order, so only a contiguous prefix counts as done */
             rel_seen[it.seq % 64] = 1;
@@ -248,7 +270,15 @@ long orc_ring_model(const size_t* call_nbytes, size_t ncalls, const int* script,
         k++;
     }
     (void)gflag;
+    if (shared_slot) *shared_slot = shared;
     return (long)k;
+}
+
+long orc_ring_model(const size_t* call_nbytes, size_t ncalls, const int* script, size_t nscript,
+                    int nslot, int nrails, size_t rail1max, int depth,
+                    uint64_t* released /* [nscript] */, int* slots /* [ncalls] */, int* rails /* [ncalls] */)
+{
+    return orc_ring_model2(call_nbytes, ncalls, script, nscript, nslot, nrails, rail1max, depth, 0, released, slots, rails, NULL);
 }
 
 /* ---------------------------------------------------------------- whole step, optionally threaded

@@ -291,6 +291,75 @@ def test_resident_peer_merged_launch_ragged(orc, streaming):
         assert not tbv.err()
 
 
+def test_early_peer_then_staged_then_early_again(orc):
+    """Early-peer mode mixed with staged calls: a staged call deposits its own payload into its receive slot, so
+    the next early-peer call that lands on that slot must get the resident payload put back (through the wire)
+    instead of summing the stale staged bytes; a full-size call restores the slot for good."""
+    nslot, n = 4, 1 << 20
+    with session(rails=2, cap=n, TBV_NSLOT=nslot) as tbv:
+        b = dev(synth.uniform(11, n // 2), torch.bfloat16)
+        tbv.peer_resident(b)
+        outs = []
+        for k in range(3 * nslot + 2):                       # slots get reused several times
+            numel = (n // 2) if k % 5 == 4 else (4096 + 512 * k)
+            a = dev(synth.uniform(100 + k, numel), torch.bfloat16)
+            out = torch.empty_like(a)
+            if k % 3 == 1:                                    # every third call brings its own payload
+                p = dev(synth.uniform(500 + k, numel), torch.bfloat16)
+                tbv.stage_peer(p)
+            else:
+                p = b[:numel]
+            assert tbv.all_reduce(a, out)
+            outs.append((k, a, p, out))
+        torch.cuda.synchronize()
+        for k, a, p, out in outs:
+            assert first_diff(out, oracle_sum(orc, a, p)) is None, k
+        assert not tbv.err()
+        tbv.peer_resident(None)
+
+
+def test_early_peer_cannot_release_a_call_still_waiting_for_rail_1(orc):
+    """A two-rail staged call whose rail-1 fragment the host holds back, followed by one-rail early-peer calls.
+    The call that wraps onto the held call's slot would raise that slot's flag on entry and so pass the held
+    call's gate while half of its receive slot is still empty; it must not be issued before the held call has
+    been released.  A second thread lifts the hold after 60 ms: the wrapping call has to have waited for it.
+    Every kernel exits normally; the held transfer is bounded by the watchdog."""
+    import threading
+    nslot, big, small = 4, 1 << 20, 8192
+    with session(rails=2, cap=big, TBV_NSLOT=nslot, TBV_WDOG=5) as tbv:
+        b = dev(synth.uniform(21, big // 2), torch.bfloat16)
+        tbv.peer_resident(b)
+        a0 = dev(synth.uniform(22, big // 2), torch.bfloat16); p0 = dev(synth.uniform(23, big // 2), torch.bfloat16)
+        o0 = torch.zeros_like(a0)
+        smalls = [dev(synth.uniform(30 + k, small // 2), torch.bfloat16) for k in range(2 * nslot)]
+        outs = [torch.empty_like(x) for x in smalls]
+        # the model: with the slot guard the host cannot issue call 1+NSLOT before rail 1 of call 1 has arrived
+        calls = [big] + [small] * nslot
+        assert orc.ring_model2(calls, [0] * (nslot + 1) + [1], nslot, 2, 98304, 0, slot_guard=1)[0] == -1
+        assert orc.ring_model2(calls, [0] * (nslot + 1) + [1], nslot, 2, 98304, 0, slot_guard=0)[4] == 1
+        torch.cuda.synchronize()
+        tbv.hold_rail(1, True)
+        tbv.stage_peer(p0)
+        assert tbv.all_reduce(a0, o0)                          # seq 1: staged, two rails, rail 1 held
+        for k in range(nslot - 1):
+            assert tbv.all_reduce(smalls[k], outs[k])          # seq 2..NSLOT: early peer, one rail, other slots
+        lifter = threading.Timer(0.06, lambda: tbv.hold_rail(1, False))
+        t0 = time.time()
+        lifter.start()
+        assert tbv.all_reduce(smalls[nslot - 1], outs[nslot - 1])   # seq 1+NSLOT wraps onto slot 1: waits for call 1's release
+        waited = time.time() - t0
+        for k in range(nslot, len(smalls)):
+            assert tbv.all_reduce(smalls[k], outs[k])
+        lifter.join()
+        torch.cuda.synchronize()
+        assert not tbv.err()
+        assert waited > 0.04, waited
+        assert first_diff(o0, oracle_sum(orc, a0, p0)) is None
+        for x, o in zip(smalls, outs):
+            assert torch.equal(o, x + b[:small // 2])
+        tbv.peer_resident(None)
+
+
 def test_full_size_properties(orc):
     """Size-independent properties at the 16 MiB bench shape: commutativity (swap local and peer),
     x + 0 = x, x + (-x) = +0, and in-place equals out-of-place."""

@@ -245,6 +245,40 @@ def test_ring_model_invariants(orc):
     assert orc.ring_model([8192], [1], 4, 2)[0] == -1             # 8 KB uses one rail only
 
 
+def test_ring_model_slot_guard(orc):
+    """A two-rail call whose rail 1 is late, followed by one-rail calls that wrap the ring.  With queue depth
+    as the only back-pressure (the reference's rule) the call that reuses the slot is issued while the slot's
+    previous user is unreleased and the two share the slot's rail counter: a release then names the wrong call.
+    (depth 0 = the host alone, no stream order: the case of calls whose flag is raised without waiting for the
+    stream because their peer payload is already there.)  Worked by hand for NSLOT = 2: calls 1 (2 rails, slot 1), 2 (slot 0), 3 (slot 1), arrivals rail 0, 0, 0, 1."""
+    big, small = 1 << 20, 8192
+    k, rel, slots, rails, shared = orc.ring_model2([big, small, small], [0, 0, 0, 1], 2, 2, 98304, 0, slot_guard=0)
+    assert k == 4 and slots == [1, 0, 1] and rails == [2, 1, 1]
+    assert shared == 1                                  # call 3 entered slot 1 while call 1 still owned it
+    assert rel == [0, 2, 3, 0]                          # call 1's rail 0 and call 3's rail 0 add up to "call 3 released":
+    assert 1 not in rel                                 # ... and call 1 is never released at all
+    # with the guard the caller holds call 3 back until call 1 is released, so rail 0 cannot arrive a third time first
+    assert orc.ring_model2([big, small, small], [0, 0, 0, 1], 2, 2, 98304, 0, slot_guard=1)[0] == -1
+    k, rel, slots, rails, shared = orc.ring_model2([big, small, small], [0, 0, 1, 0], 2, 2, 98304, 0, slot_guard=1)
+    assert k == 4 and shared == 0 and rel == [0, 2, 1, 3]
+    # seeded mixes: the guard never lets two calls share a slot and every call is released exactly once, by its own last rail
+    for seed in range(20):
+        r = synth.bits32(9100 + seed, 40, 3)
+        calls = [big if int(v) % 3 == 0 else small for v in r]
+        script = []
+        nslot = 2 + seed % 3
+        order = synth.bits32(9200 + seed, 80, 5)
+        # a script that is legal under the guard: arrivals in call order, the two rails of a call in seeded order
+        for i, nb in enumerate(calls):
+            rs = [0, 1] if nb == big else [0]
+            if nb == big and int(order[i]) & 1:
+                rs = [1, 0]
+            script += rs
+        k, rel, slots, rails, shared = orc.ring_model2(calls, script, nslot, 2, 98304, 0, slot_guard=1)
+        assert k == len(script) and shared == 0
+        assert sorted(x for x in rel if x) == list(range(1, len(calls) + 1))
+
+
 def test_whole_step_threaded_equals_single(orc):
     n = 300001
     a = tbits(torch.from_numpy(synth.uniform(1, n)).to(torch.bfloat16)).copy()
