@@ -181,6 +181,24 @@ void tbv_emu_shutdown(void);
  * Same return codes as tbv_ar_allreduce, except that no size is over the cap. */
 int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, int dtype, void* stream);
 
+/* The all-reduce followed by the RMSNorm of its result in one pass over the hidden state.
+ * The reference plans this fusion but does not have it (reports/12_references.md:136:
+ * the all-reduce tail k_acc fused with the next RMSNorm); the arithmetic is that of the
+ * fused add + RMSNorm of its caller (vLLM): with T the storage type,
+ *   out    = ptr + peer                      (as tbv_ar_allreduce, bit for bit; outp NULL = in place)
+ *   normed = T(float(out) * s) * weight      (product in T), s = 1 / sqrt(mean(float(out)^2 over a row) + eps)
+ * for `rows` rows of `hidden` elements; `weight` holds `hidden` elements of T.  The sum of
+ * squares is taken in fp32 in a fixed order, so results are reproducible.  A row must be a
+ * multiple of 16 bytes and at most 64 KiB, and all buffers 16-byte aligned (-1 otherwise).
+ * Return codes as tbv_ar_allreduce (-2: rows * hidden exceeds the cap). */
+int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, const void* weight, float eps,
+                             size_t rows, size_t hidden, int dtype, void* stream);
+
+/* Standalone row kernel for benches and tests: mode 0: normed = rmsnorm(a) * weight;
+ * mode 1: out = a + b, normed = rmsnorm(out) * weight. */
+int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const void* b, void* normed, const void* weight, float eps,
+                         size_t rows, size_t hidden, int dtype, void* stream);
+
 /* Standalone kernel entry points for benches and tests: run only the pack copy
  * (into send slot `slot`, with completion signal) or only the sum, on `stream`. */
 int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream);

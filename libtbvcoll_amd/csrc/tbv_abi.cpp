@@ -245,6 +245,48 @@ extern "C" int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, in
     return 0;
 }
 
+// The all-reduce followed by the RMSNorm of its result, in one pass over the hidden state (planned, not built,
+// in the reference: reports/12_references.md:136).
+extern "C" int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, const void* weight, float eps,
+                                        size_t rows, size_t hidden, int dtype, void* stream)
+{
+    if (!G.inited) FAIL("not initialised");
+    if (G.err.load(std::memory_order_relaxed)) FAIL("an earlier transfer failed; the library cannot recover");
+    if (dtype < 0 || dtype > 2) FAIL("unknown dtype %d", dtype);
+    const size_t esz = dtype == 0 ? 4 : 2;
+    if (rows == 0 || hidden == 0) return 0;
+    if (hidden > ((size_t)1 << 40) / rows) return -2;
+    const size_t nbytes = rows * hidden * esz;
+    if (nbytes > G.cap) return -2;                    // caller falls back to its own collective and norm
+    if (!row_norm_shape_ok(rows, hidden, dtype)) FAIL("rmsnorm rows must be a multiple of 16 bytes and at most %d bytes", kRowNormMaxVecs * 16);
+    if (!normed || !weight || !ptr) FAIL("null buffer");
+    if (!outp) outp = ptr;
+    if (((uintptr_t)ptr | (uintptr_t)outp | (uintptr_t)normed | (uintptr_t)weight) & 15) FAIL("rmsnorm buffers must be 16-byte aligned");
+    if (G.async && !G.run.load(std::memory_order_relaxed)) FAIL("progress threads were stopped by tbv_ar_fini");
+    hipStream_t st = (hipStream_t)stream;
+    note_stream(stream, nbytes);
+    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
+    const double te = nowt();
+    Call c;
+    if (enqueue_pack(ptr, outp, nbytes, dtype, st, &c, &nm) != 0) return -1;
+    if (enqueue_wait_sum(ptr, outp, dtype, st, c, &nm) != 0) return -1;
+    if (flush_pending() != 0) FAIL("deferred signal launch failed");
+    G.t_enq += nowt() - te;
+    return 0;
+}
+
+// Standalone row kernel for benches and tests: mode 0 normalises `a`; mode 1 writes out = a + b and normalises it.
+extern "C" int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const void* b, void* normed, const void* weight, float eps,
+                                    size_t rows, size_t hidden, int dtype, void* stream)
+{
+    if (dtype < 0 || dtype > 2 || mode < 0 || mode > 1 || !row_norm_shape_ok(rows, hidden, dtype)) return -1;
+    const size_t esz = dtype == 0 ? 4 : 2;
+    SumArgs sa{};
+    sa.out = out; sa.a = a; sa.b = b; sa.nbytes = rows * hidden * esz; sa.dtype = dtype;
+    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
+    return launch_row_norm(mode, nullptr, sa, nm, (hipStream_t)stream) == hipSuccess ? 0 : -1;
+}
+
 extern "C" int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream)
 {
     if (!G.inited || slot < 0 || slot >= G.nslot || nbytes > G.cap) return -1;

@@ -295,7 +295,7 @@ int configure(const char* devs, size_t cap)
 
 // First half of a call: sequence number, slot, pack kernel, work items.
 // `sum_out`/`dtype` are only used when the sum can share the pack's launch.
-int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c)
+int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm)
 {
     const size_t tagoff = tag_offset(nbytes);
     c->nbytes = nbytes;
@@ -324,14 +324,14 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         if (G.gpusig) {
             const bool aligned = !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
             const bool plain = sum_out && !G.tag && G.kwait != 1 && !(G.railsum && c->R > 1) && aligned;
-            const bool can_fuse = G.fuse && c->resident && plain;
+            const bool can_fuse = G.fuse && c->resident && plain && !nm;
             // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
             // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
             const bool one_kernel = G.onekernel && !can_fuse && plain && G.can_wait_value && nbytes <= G.fusewait_max &&
-                                    small_call_blocks(nbytes) <= kSmallCallMaxBlocks;
+                                    (nm ? nm->rows <= (unsigned)kRowNormMaxSmallRows : small_call_blocks(nbytes) <= kSmallCallMaxBlocks);
             // Payload already in place and too large for the one-kernel call: pack blocks and sum blocks in one
             // launch (a launch costs about 2.4 us of stream time whatever it does).
-            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && plain && G.packsig == 0;
+            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && plain && G.packsig == 0 && !nm;
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
@@ -356,7 +356,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (G.probe.load(std::memory_order_relaxed)) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
                 KTimer kt(1);
                 const double tq = nowt();
-                const hipError_t e = one_kernel ? launch_small_call(pa, sa, st, kt.get())
+                const hipError_t e = one_kernel ? (nm ? launch_row_norm(2, &pa, sa, *nm, st, kt.get()) : launch_small_call(pa, sa, st, kt.get()))
                                    : can_fuse ? launch_pack_sum(pa, sa, st, kt.get()) : launch_pack_sum_merged(pa, sa, st, kt.get());
                 if (e != hipSuccess) FAIL("%s launch failed", one_kernel ? "one-kernel call" : "pack+sum kernel");
                 G.t_post += nowt() - tq;                       // the launch that carries the sum
@@ -399,7 +399,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
 }
 
 // Second half: gate the stream on the flag(s), then the sum.
-int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c)
+int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm)
 {
     if (c.fused) return 0;
     const char* rb = slot_recv(c.slot);
@@ -416,7 +416,10 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         if (probe && last) { sa.done = doneword(c.slot); sa.done_arrive = done_counters(c.slot); }
         sa.pre = take_pending(st);
         KTimer kt(1);
-        if (launch_sum(sa, st, kt.get()) != hipSuccess) FAIL("sum kernel launch failed");
+        // with a norm to follow and the whole payload in this piece, the sum kernel is the row kernel that also normalises
+        const bool with_norm = nm && off == 0 && len == c.nbytes;
+        if ((with_norm ? launch_row_norm(1, nullptr, sa, *nm, st, kt.get()) : launch_sum(sa, st, kt.get())) != hipSuccess)
+            FAIL("sum kernel launch failed");
         return 0;
     };
     auto gate_stream = [&](unsigned long long* flag) -> int {
@@ -443,11 +446,18 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
             if (off + len >= c.nbytes) l = ((c.nbytes - off) / esz) * esz;
             if (sum_piece(off, l, nullptr, pieces == total) != 0) return -1;
         }
+        if (nm) {                            // per-rail sums cannot normalise whole rows: normalise the finished output
+            SumArgs sa{};
+            sa.a = outp; sa.nbytes = c.nbytes; sa.dtype = dtype; sa.seq = c.seq;
+            if (launch_row_norm(0, nullptr, sa, *nm, st) != hipSuccess) FAIL("norm kernel launch failed");
+        }
     } else {
         // The flag may already be up when the call is made (the peer was early): the payload is then in
         // place before the sum is even launched and the stream needs no gate at all.
         const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
-        const bool fusewait = G.async && !arrived && (c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1;
+        // (a row kernel has one block per row and no grid cap: it may only wait inside when its rows are few)
+        const bool fusewait = G.async && !arrived && (c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
+                              !(nm && nm->rows > (unsigned)kRowNormMaxSmallRows);
         if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
             if (launch_tagchk((const unsigned long long*)(rb + tag_offset(c.nbytes)), c.seq, dbgwords(), st) != hipSuccess)

@@ -192,8 +192,8 @@ int configure(const char* devs, size_t cap);
 int init_impl(int rank, const char* devs, size_t cap);
 void teardown();
 void stop_progress();
-int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c);
-int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c);
+int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm = nullptr);
+int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm = nullptr);
 int flush_pending();
 void note_stream(void* stream, size_t nbytes);
 bool rails_idle();

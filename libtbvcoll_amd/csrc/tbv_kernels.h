@@ -83,6 +83,21 @@ hipError_t launch_tagchk(const unsigned long long* tag, unsigned long long seq, 
 hipError_t launch_mark(unsigned long long* fp, int i, unsigned long long seq, hipStream_t st);
 hipError_t launch_fill_u32(unsigned int* p, unsigned int v, size_t n, hipStream_t st);
 
+// Row-wise RMSNorm fused with the sum (tbv_norm.hip).  A row is `row_vecs` 16-byte vectors; `weight` holds one row.
+struct NormArgs {
+    const void* weight;
+    void* normed;
+    float eps;
+    unsigned row_vecs;
+    unsigned rows;
+};
+static constexpr int kRowNormMaxVecs = 4096;          // 64 KiB per row: 1024 lanes x 4 vectors
+static constexpr int kRowNormMaxSmallRows = 128;      // one-launch form: every block must be resident while it waits
+bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype);
+// mode 0: normed = rmsnorm(s.a) * weight.   mode 1: out = a + b (s.wait_flag optional), normed = rmsnorm(out) * weight.
+// mode 2: the whole small call in one launch (pack `p`, completion word, flag poll, sum, norm).
+hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& s, const NormArgs& n, hipStream_t st, const Timing* t = nullptr);
+
 // Looks up this device's copy of the built-in counter array of tbv_step_noalloc (once per device).
 bool noalloc_bind_device();
 

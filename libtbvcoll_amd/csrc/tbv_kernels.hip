@@ -11,199 +11,9 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include "tbv_kernels.h"
+#include "tbv_device.h"
 
 namespace tbv {
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-// Cache hints of the four data streams, two profiles measured on MI355X with the 16 MiB step.
-//
-// Resident profile (STREAM = false): what a step touches stays in the 256 MB Infinity Cache
-// (small rings, the same tensors every step).  The local tensor is read twice (pack, then
-// sum) and the receive slots are re-read every NSLOT calls, so both are left to allocate in
-// the caches; the output is written once and never read here, so it is stored non-temporally
-// and leaves the cache to the operands (sum 7.6 -> 6.6 us); the uncached bounce gets no hint.
-// Non-temporal loads of the local tensor or the receive slot cost 1-2 us per step here.
-//
-// Streaming profile (STREAM = true): the rings are larger than the cache, every operand
-// comes from HBM and nothing written is read again soon.  The receive slot is loaded and
-// the bounce and the output are stored non-temporally; the local tensor keeps ordinary
-// loads because the sum re-reads it a few microseconds after the pack, except in the fused
-// kernel, its only reader (pack + sum
-// 15.98 -> 14.18 us on cache-cold buffers; the same hints cost 0.3 us when everything is
-// cache resident, which is why there are two profiles).
-// ONCE: this kernel is the only reader of the local tensor (pack and sum fused in one body)
-template <bool STREAM, bool ONCE> __device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_a(const uint32_t __attribute__((ext_vector_type(4)))* p)
-{
-    return *p;          // non-temporal here costs about 1 us per 16 MiB even when this kernel is the only reader
-}
-template <bool STREAM> __device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4))) ld_b(const uint32_t __attribute__((ext_vector_type(4)))* p)
-{
-    return STREAM ? __builtin_nontemporal_load(p) : *p;
-}
-template <bool STREAM> __device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
-{
-    __builtin_nontemporal_store(v, p);
-}
-template <bool STREAM> __device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
-{
-    if (STREAM) __builtin_nontemporal_store(v, p); else *p = v;
-}
-
-static constexpr int kThreads = 256;        // 4 wavefronts of 64
-static constexpr int kMaxSmallThreads = 1024;
-static constexpr int kMaxGrid = 256 * 8;     // 256 CUs, up to 8 resident blocks each
-// A kernel that waits for the flag inside holds its wave slots while it waits.  Whatever has to
-// run for the flag to come up (another stream's copy, another library's kernel) needs slots too,
-// so a gated grid is kept to an eighth of the GPU's 8192 wave slots; the blocks loop instead.
-static constexpr int kGatedMaxGrid = 256;
-
-// ---------------------------------------------------------------- arithmetic
-
-// bf16: widen both operands to fp32 (exact), add in fp32, round to nearest even.
-// The fptrunc of a float pair lowers to v_cvt_pk_bf16_f32 on gfx950.
-__device__ __forceinline__ uint32_t add_bf16x2(uint32_t x, uint32_t y)
-{
-    f32x2 s;
-    s.x = __uint_as_float(x << 16) + __uint_as_float(y << 16);
-    s.y = __uint_as_float(x & 0xffff0000u) + __uint_as_float(y & 0xffff0000u);
-    bf16x2 r = __builtin_convertvector(s, bf16x2);
-    return __builtin_bit_cast(uint32_t, r);
-}
-
-template <int DT> __device__ __forceinline__ u32x4 add_vec(u32x4 x, u32x4 y);
-
-template <> __device__ __forceinline__ u32x4 add_vec<0>(u32x4 x, u32x4 y)
-{
-    f32x4 a = __builtin_bit_cast(f32x4, x), b = __builtin_bit_cast(f32x4, y);
-    f32x4 s;
-    s.x = a.x + b.x; s.y = a.y + b.y; s.z = a.z + b.z; s.w = a.w + b.w;
-    return __builtin_bit_cast(u32x4, s);
-}
-// fp16: the IEEE half add itself (what the HIP header's operator+ on _Float16 is);
-// it equals fp32-upcast + add + round-to-nearest-even for every finite pair.
-template <> __device__ __forceinline__ u32x4 add_vec<1>(u32x4 x, u32x4 y)
-{
-    f16x8 a = __builtin_bit_cast(f16x8, x), b = __builtin_bit_cast(f16x8, y);
-    f16x8 s = a + b;
-    return __builtin_bit_cast(u32x4, s);
-}
-template <> __device__ __forceinline__ u32x4 add_vec<2>(u32x4 x, u32x4 y)
-{
-    u32x4 r;
-    r.x = add_bf16x2(x.x, y.x); r.y = add_bf16x2(x.y, y.y);
-    r.z = add_bf16x2(x.z, y.z); r.w = add_bf16x2(x.w, y.w);
-    return r;
-}
-
-template <int DT> struct Elem;
-template <> struct Elem<0> { typedef float T; static __device__ __forceinline__ T add(T a, T b) { return a + b; } };
-template <> struct Elem<1> { typedef _Float16 T; static __device__ __forceinline__ T add(T a, T b) { return a + b; } };
-template <> struct Elem<2> {
-    typedef uint16_t T;
-    static __device__ __forceinline__ T add(T a, T b)
-    {
-        float s = __uint_as_float((uint32_t)a << 16) + __uint_as_float((uint32_t)b << 16);
-        __bf16 r = (__bf16)s;
-        return __builtin_bit_cast(uint16_t, r);
-    }
-};
-
-// ---------------------------------------------------------------- signalling helpers
-
-__device__ __forceinline__ void store_sys(unsigned long long* p, unsigned long long v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-}
-
-// Every thread of the block calls this after its last store.  `bid` of `nblk` is the
-// block's index among the blocks being counted (the whole grid, or one part of a merged
-// launch).  When the last of them gets here, all their stores are visible system wide
-// and `word` is set to `seq`.
-//
-// Blocks are counted in two levels so that no single address takes one atomic
-// per block (same-address atomics retire one at a time): groups of kGroup blocks
-// count on their own 64-byte line, and the last block of a group counts on the
-// top line.  `ctr` points to the slot's counter lines (line 0 = top, line 1+g =
-// group g, 16 words apart); every counter is put back to 0 by its last arriver.
-//
-// mode 0: the destination is uncached memory: stores bypass the L2, so each wave
-//         only has to see its own stores acknowledged before the block is counted.
-//         (The workgroup-scope release inside __syncthreads does not wait for the
-//         store counter on gfx950, hence the explicit wait.)
-// mode 1: the destination may be cached: the block leader also writes the L2 back
-//         system wide after the barrier (one write-back per block).
-// mode 2: every wave writes back system wide before the barrier (most conservative).
-static constexpr unsigned kGroup = 32;
-static constexpr unsigned kCtrLine = 16;       // words per counter line (64 bytes)
-
-__device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
-                                              unsigned int* ctr, unsigned int bid, unsigned int nblk, int mode)
-{
-    if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        if (mode == 1) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-        bool last = true;
-        if (nblk > 1) {
-            const unsigned g = bid / kGroup, ngroups = (nblk + kGroup - 1) / kGroup;
-            const unsigned pop = min(kGroup, nblk - g * kGroup);
-            unsigned int* gc = ctr + kCtrLine * (1 + g);
-            last = false;
-            if (__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == pop - 1) {
-                __hip_atomic_store(gc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (ngroups == 1) last = true;
-                else if (__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1) {
-                    __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    last = true;
-                }
-            }
-        }
-        if (last) store_sys(word, seq);
-    }
-}
-
-// Gate of a kernel on a host-visible word reaching seq.  Only block 0's leader
-// polls the host word (each poll crosses PCIe); it republishes the value in a
-// device word (`relay`) that the other blocks' leaders poll at L2 latency.  Block
-// 0 never waits on another block, so the gate cannot deadlock however many blocks
-// are resident.  Every wait is bounded by a tick count of the constant-rate wall
-// clock (100 MHz on gfx950; the host passes ticks computed from the device's
-// reported rate), so every wave leaves the kernel even if nobody raises the word.
-__device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsigned long long seq,
-                                          unsigned long long limit, unsigned long long* relay,
-                                          unsigned long long* fp)
-{
-    if (threadIdx.x == 0) {
-        const unsigned long long t0 = wall_clock64();
-        if (blockIdx.x == 0 || !relay) {
-            if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_IN, seq);
-            // relaxed polls: an acquire load in the loop would invalidate the caches on every iteration, for this
-            // kernel and for whatever is writing the payload; one acquire fence follows the barrier below
-            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
-                __builtin_amdgcn_s_sleep(1);
-                if (wall_clock64() - t0 > limit) {
-                    if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
-                    break;
-                }
-            }
-            if (relay) __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-            if (fp && blockIdx.x == 0) store_sys(fp + FP_WAIT_OUT, seq);
-        } else {
-            while (__hip_atomic_load(relay, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < seq) {
-                __builtin_amdgcn_s_sleep(2);
-                if (wall_clock64() - t0 > limit + limit / 8 + 1000000ull) break;
-            }
-        }
-    }
-    __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");       // the payload was written before the flag: no stale lines from here on
-}
 
 // ---------------------------------------------------------------- the step kernel
 //
@@ -212,18 +22,6 @@ __device__ __forceinline__ void gate_wait(const unsigned long long* flag, unsign
 // U loads of a lane blockDim vectors apart, so each wavefront instruction touches
 // 1 KiB of consecutive memory and a lane has U (x2 for the sum) loads in flight.
 
-struct StepArgs {
-    // pack
-    u32x4* bounce; unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long* tagp;
-    // sum
-    u32x4* out; const u32x4* b;
-    const unsigned long long* wait_flag; unsigned long long* relay; unsigned long long spin_limit;
-    unsigned long long* done; unsigned int* done_arrive;
-    // common
-    const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp; int sigmode;
-    unsigned long long* pre_word; unsigned long long pre_seq;
-    unsigned pack_blocks;       // merged launch: blocks [0, pack_blocks) pack, the rest sum
-};
 
 // Block `bid` of `nblk` does its share of the payload; block 0 also does the bytes past the last whole vector.
 template <int DT, int U, bool PACK, bool SUM, bool STREAM>

@@ -1,0 +1,213 @@
+// All-reduce tail fused with the RMSNorm that follows it: one pass over the hidden state
+// writes both the reduced tensor (the residual stream) and its normalised form.
+//
+// The reference only plans this ("k_acc + next RMSNorm in one kernel: one launch and one
+// hidden-state read/write less, 56 times per step", reports/12_references.md:136).  The
+// arithmetic follows the fused add + RMSNorm of the reference's caller (vLLM's
+// fused_add_rms_norm): z = local + received rounded to the storage type (exactly the sum
+// kernel's result, step4/libtbvcoll.cpp:162-166), x = float(z), s = 1 / sqrt(mean(x^2) + eps),
+// normed = T(x * s) * weight with the product taken in the storage type.
+//
+// One block per row.  Lane t of L holds vectors t, t+L, ... of the row in registers, so the
+// row is read once; the sum of squares is accumulated with fused multiply-adds in a fixed
+// order (per lane: its vectors in order, elements in order; per wave: xor butterfly 32, 16,
+// 8, 4, 2, 1; per block: the waves' totals in wave order), which makes the result
+// reproducible and lets a CPU restatement match it bit for bit.  1/sqrt is the correctly
+// rounded division of the correctly rounded square root.
+//
+// MODE 0: normalise `a` as it is (no sum; used after an all-reduce that ran unfused)
+// MODE 1: z = a + b, write z to out, normalise z
+// MODE 2: the whole small call in one launch: pack a into the bounce slot, count the blocks and
+//         raise the pack's completion word, poll the flag, then as MODE 1 (grid small enough
+//         for all blocks to be resident together, as for k_small_call)
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include "tbv_device.h"
+#include "tbv_kernels.h"
+
+namespace tbv {
+
+namespace {
+
+template <int DT> struct Row;
+// f32: 4 elements per vector
+template <> struct Row<0> {
+    static constexpr int EPV = 4;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+    }
+    static __device__ __forceinline__ u32x4 scale(u32x4 v, u32x4 w, float s)
+    {
+        float f[4], g[4]; unpack(v, f); unpack(w, g);
+        u32x4 r;
+        r.x = __float_as_uint((f[0] * s) * g[0]); r.y = __float_as_uint((f[1] * s) * g[1]);
+        r.z = __float_as_uint((f[2] * s) * g[2]); r.w = __float_as_uint((f[3] * s) * g[3]);
+        return r;
+    }
+};
+// f16: 8 elements per vector; T(x*s) by round-to-nearest-even conversion, then the half multiply
+template <> struct Row<1> {
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        f16x8 h = __builtin_bit_cast(f16x8, v);
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ u32x4 scale(u32x4 v, u32x4 w, float s)
+    {
+        f16x8 h = __builtin_bit_cast(f16x8, v), g = __builtin_bit_cast(f16x8, w), r;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { _Float16 t = (_Float16)((float)h[i] * s); r[i] = t * g[i]; }
+        return __builtin_bit_cast(u32x4, r);
+    }
+};
+// bf16: 8 elements per vector; both roundings to nearest even from fp32
+template <> struct Row<2> {
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) { f[2 * i] = __uint_as_float(u[i] << 16); f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u); }
+    }
+    static __device__ __forceinline__ uint32_t bf16(float x)
+    {
+        __bf16 r = (__bf16)x;
+        return (uint32_t)__builtin_bit_cast(uint16_t, r);
+    }
+    static __device__ __forceinline__ u32x4 scale(u32x4 v, u32x4 w, float s)
+    {
+        float f[8], g[8]; unpack(v, f); unpack(w, g);
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float t0 = __uint_as_float(bf16(f[2 * i] * s) << 16), t1 = __uint_as_float(bf16(f[2 * i + 1] * s) << 16);
+            o[i] = bf16(t0 * g[2 * i]) | (bf16(t1 * g[2 * i + 1]) << 16);
+        }
+        u32x4 r = {o[0], o[1], o[2], o[3]};
+        return r;
+    }
+};
+
+template <int DT, int VPL, int MODE>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormArgs nm)
+{
+    __shared__ float wave_total[kMaxSmallThreads / 64];
+    const unsigned tid = threadIdx.x, lanes = blockDim.x, hv = nm.row_vecs;
+    const size_t row0 = (size_t)blockIdx.x * hv;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (MODE == 2 && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+
+    u32x4 x[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {
+        const unsigned j = tid + (unsigned)v * lanes;
+        const u32x4 zero = {0, 0, 0, 0};
+        x[v] = j < hv ? g.a[row0 + j] : zero;
+        if (MODE == 2 && j < hv) g.bounce[row0 + j] = x[v];
+    }
+    if (MODE == 2) {
+        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
+        if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    } else if (MODE == 1 && g.wait_flag) {
+        gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    }
+    float ssq = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {
+        const unsigned j = tid + (unsigned)v * lanes;
+        if (MODE >= 1 && j < hv) {
+            x[v] = add_vec<DT>(x[v], g.b[row0 + j]);
+            __builtin_nontemporal_store(x[v], g.out + row0 + j);
+        }
+        float f[Row<DT>::EPV];
+        Row<DT>::unpack(x[v], f);                            // lanes past the row hold zeros: they add nothing
+#pragma unroll
+        for (int e = 0; e < Row<DT>::EPV; e++) ssq = __builtin_fmaf(f[e], f[e], ssq);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+    if ((tid & 63) == 0) wave_total[tid >> 6] = ssq;
+    __syncthreads();
+    float total = wave_total[0];
+    for (unsigned w = 1; w < (lanes >> 6); w++) total += wave_total[w];
+    const float s = 1.0f / __builtin_sqrtf(total / (float)((size_t)hv * Row<DT>::EPV) + nm.eps);
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {
+        const unsigned j = tid + (unsigned)v * lanes;
+        if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], ((const u32x4*)nm.weight)[j], s), (u32x4*)nm.normed + row0 + j);
+    }
+    if (MODE >= 1 && g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+}
+
+template <typename A, typename B>
+hipError_t launch2(void (*kernel)(A, B), int grid, int block, hipStream_t st, const Timing* t, const A& a, const B& b)
+{
+    if (t && t->start && t->stop) hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, t->start, t->stop, 0, a, b);
+    else hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, a, b);
+    return hipGetLastError();
+}
+
+template <int DT, int MODE>
+hipError_t launch_vpl(int vpl, int grid, int block, hipStream_t st, const Timing* t, const StepArgs& s, const NormArgs& n)
+{
+    switch (vpl) {
+        case 1: return launch2(k_row_norm<DT, 1, MODE>, grid, block, st, t, s, n);
+        case 2: return launch2(k_row_norm<DT, 2, MODE>, grid, block, st, t, s, n);
+        default: return launch2(k_row_norm<DT, 4, MODE>, grid, block, st, t, s, n);
+    }
+}
+
+template <int MODE>
+hipError_t launch_dt(int dtype, int vpl, int grid, int block, hipStream_t st, const Timing* t, const StepArgs& s, const NormArgs& n)
+{
+    switch (dtype) {
+        case 0: return launch_vpl<0, MODE>(vpl, grid, block, st, t, s, n);
+        case 1: return launch_vpl<1, MODE>(vpl, grid, block, st, t, s, n);
+        case 2: return launch_vpl<2, MODE>(vpl, grid, block, st, t, s, n);
+    }
+    return hipErrorInvalidValue;
+}
+
+inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+}  // namespace
+
+bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype)
+{
+    const size_t esz = dtype == 0 ? 4 : 2, row_bytes = hidden * esz;
+    return rows >= 1 && rows <= 0x7fffffffu && hidden >= 1 && (row_bytes & 15) == 0 && (row_bytes >> 4) <= (size_t)kRowNormMaxVecs;
+}
+
+hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const NormArgs& nm, hipStream_t st, const Timing* t)
+{
+    if (mode < 0 || mode > 2 || q.dtype < 0 || q.dtype > 2 || !nm.weight || !nm.normed || !q.a) return hipErrorInvalidValue;
+    const size_t esz = q.dtype == 0 ? 4 : 2;
+    if (!nm.rows || !nm.row_vecs || nm.row_vecs > (unsigned)kRowNormMaxVecs || q.nbytes != (size_t)nm.rows * nm.row_vecs * 16) return hipErrorInvalidValue;
+    if (!(al16(q.a) && al16(nm.weight) && al16(nm.normed))) return hipErrorInvalidValue;
+    if (mode >= 1 && (!q.out || !q.b || !al16(q.out) || !al16(q.b) || (q.done && !q.done_arrive))) return hipErrorInvalidValue;
+    if (mode == 2 && (!p || !p->dst || !al16(p->dst) || !p->cflag || !p->arrive || p->src != q.a || p->nbytes != q.nbytes ||
+                      nm.rows > (unsigned)kRowNormMaxSmallRows)) return hipErrorInvalidValue;
+    (void)esz;
+    StepArgs s{};
+    if (mode == 2) { s.bounce = (u32x4*)p->dst; s.cflag = p->cflag; s.pack_arrive = p->arrive; s.sigmode = p->sigmode; s.fp = p->fp;
+                     s.pre_word = p->pre.word; s.pre_seq = p->pre.seq; }
+    else { s.pre_word = q.pre.word; s.pre_seq = q.pre.seq; s.fp = q.fp; }
+    s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.done = q.done; s.done_arrive = q.done_arrive;
+    s.a = (const u32x4*)q.a; s.nbytes = q.nbytes; s.seq = q.seq;
+    int vpl = (int)((nm.row_vecs + kMaxSmallThreads - 1) / kMaxSmallThreads);
+    vpl = vpl <= 1 ? 1 : vpl == 2 ? 2 : 4;
+    int block = (int)(((nm.row_vecs + vpl - 1) / vpl + 63) / 64 * 64);
+    const int grid = (int)nm.rows;
+    switch (mode) {
+        case 0: return launch_dt<0>(q.dtype, vpl, grid, block, st, t, s, nm);
+        case 1: return launch_dt<1>(q.dtype, vpl, grid, block, st, t, s, nm);
+        default: return launch_dt<2>(q.dtype, vpl, grid, block, st, t, s, nm);
+    }
+}
+
+}  // namespace tbv

@@ -55,6 +55,8 @@ _SIGNATURES = {
     "tbv_emu_run_pack": (_I, [_VP, _SZ, _I, _VP]), "tbv_emu_run_sum": (_I, [_VP, _VP, _VP, _SZ, _I, _VP]),
     "tbv_step_noalloc": (_I, [_VP, _VP, _VP, _VP, _I, _SZ, _I, _VP, _VP, _U64, _VP]),
     "tbv_emu_hbm_probe": (_I, [_I, _SZ, _SZ, _I, _PD, _PD]), "tbv_emu_launch_floor": (_I, [_I, _PD]),
+    "tbv_ar_allreduce_rmsnorm": (_I, [_VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
+    "tbv_emu_run_sum_norm": (_I, [_I, _VP, _VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
 }
 
 
@@ -295,6 +297,30 @@ def all_reduce_chunked(t: torch.Tensor, out: torch.Tensor = None) -> bool:
     pin, pout, nb, code = a
     _check(_lib.tbv_ar_allreduce_chunked(pin, pout, nb, code, _stream()), "tbv_ar_allreduce_chunked")
     return True
+
+
+def all_reduce_rmsnorm(t: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor = None, normed: torch.Tensor = None):
+    """SUM with the peer fused with the RMSNorm of the result over the last dimension:
+    out = t + peer (in place when out is None), normed = rmsnorm(out) * weight.  Returns `normed`
+    (allocated when not given), or None when the library does not take the call (not initialised,
+    unsupported layout, over the cap): the caller then runs its own all-reduce and norm."""
+    a = _call_args(t, out)
+    if a is None or t.dim() < 1 or weight.dtype is not t.dtype or not weight.is_contiguous() or weight.numel() != t.shape[-1]:
+        return None
+    pin, pout, nb, code = a
+    if nb == 0 or nb > _cap:
+        return None
+    hidden = t.shape[-1]
+    if normed is None:
+        normed = torch.empty_like(t)
+    elif not normed.is_contiguous() or normed.dtype is not t.dtype or normed.numel() != t.numel():
+        return None
+    rc = _lib.tbv_ar_allreduce_rmsnorm(pin, pout, _VP(normed.data_ptr()), _VP(weight.data_ptr()), eps,
+                                       t.numel() // hidden, hidden, code, _stream())
+    if rc == -2:
+        return None
+    _check(rc, "tbv_ar_allreduce_rmsnorm")
+    return normed
 
 
 def shutdown():

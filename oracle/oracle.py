@@ -57,6 +57,8 @@ def lib():
         l.orc_ring_model2.argtypes = [ctypes.POINTER(sz), sz, ctypes.POINTER(ci), sz, ci, ci, sz, ci, ci,
                                       ctypes.POINTER(u64), ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ctypes.c_long)]
         l.orc_ring_model2.restype = ctypes.c_long
+        l.orc_rmsnorm_rows.argtypes = [ci, vp, vp, vp, sz, sz, ctypes.c_float]; l.orc_rmsnorm_rows.restype = ci
+        l.orc_sum_rmsnorm.argtypes = [ci, vp, vp, vp, vp, vp, sz, sz, ctypes.c_float]; l.orc_sum_rmsnorm.restype = ci
         l.orc_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci]; l.orc_reduce_copy.restype = ci
         l.orc_time_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci, ci, ci]; l.orc_time_reduce_copy.restype = ctypes.c_double
         _lib = l
@@ -132,6 +134,27 @@ def ring_model2(call_nbytes, script, nslot, nrails, rail1max=98304, depth=1, slo
     shared = ctypes.c_long(0)
     k = lib().orc_ring_model2(calls, n, scr, m, nslot, nrails, rail1max, depth, slot_guard, rel, slots, rails, ctypes.byref(shared))
     return k, list(rel)[:max(k, 0)], list(slots)[:n], list(rails)[:n], shared.value
+
+
+def rmsnorm_rows(dtype, x, w, hidden, eps):
+    """normed = T(float(x) * s) * w per row of `hidden` elements, s = 1/sqrt(mean(x^2) + eps); storage-bit arrays."""
+    x = np.ascontiguousarray(x, dtype=_NP[dtype]).reshape(-1); w = np.ascontiguousarray(w, dtype=_NP[dtype]).reshape(-1)
+    assert w.size == hidden and x.size % hidden == 0
+    out = np.empty_like(x)
+    rc = lib().orc_rmsnorm_rows(dtype, _p(x), _p(w), _p(out), x.size // hidden, hidden, eps)
+    assert rc == 0
+    return out
+
+
+def sum_rmsnorm(dtype, a, b, w, hidden, eps):
+    """(out, normed) of the fused step: out = a + b in the storage type, normed = rmsnorm(out) * w."""
+    a = np.ascontiguousarray(a, dtype=_NP[dtype]).reshape(-1); b = np.ascontiguousarray(b, dtype=_NP[dtype]).reshape(-1)
+    w = np.ascontiguousarray(w, dtype=_NP[dtype]).reshape(-1)
+    assert a.size == b.size and w.size == hidden and a.size % hidden == 0
+    out = np.empty_like(a); normed = np.empty_like(a)
+    rc = lib().orc_sum_rmsnorm(dtype, _p(a), _p(b), _p(w), _p(out), _p(normed), a.size // hidden, hidden, eps)
+    assert rc == 0
+    return out, normed
 
 
 def reduce_copy(dtype, local, peer, nthreads=1):

@@ -349,3 +349,105 @@ double orc_time_reduce_copy(int dtype, const void* local, const void* peer, void
     free(t);
     return med;
 }
+
+/* ---------------------------------------------------------------- sum + RMSNorm in one pass
+ * The reference only plans this fusion (reports/12_references.md:136: "k_acc + the next RMSNorm");
+ * the arithmetic restated here is the fused add + RMSNorm of its caller, vLLM's fused_add_rms_norm:
+ *   z = a + b rounded to the storage type (orc_sum above, step4/libtbvcoll.cpp:162-166)
+ *   x = float(z);  s = 1 / sqrt(mean(x^2) + eps);  normed = T(x * s) * w, the product taken in T.
+ * fp32 addition is not associative, so the order of the sum of squares is part of the definition.
+ * The order below is the one the GPU kernel documents: a row of `hidden` elements is cut into
+ * 16-byte vectors; with L = lanes (a multiple of 64) lane t accumulates, by fused multiply-add,
+ * the elements of vectors t, t+L, t+2L, ... in index order; each 64-lane wave is reduced by the
+ * xor butterfly 32,16,8,4,2,1; the waves' totals are added in wave order.  1/sqrt is the
+ * correctly rounded division of the correctly rounded square root.  L follows from the row:
+ * vpl = ceil(vectors / 1024) rounded up to 1, 2 or 4; L = ceil(vectors / vpl) rounded up to 64.
+ * Pinned in the tests against torch's fp32 formula (x.float().pow(2).mean(-1), rsqrt) within 2 ulp
+ * of T, and against closed-form rows.
+ */
+#include <math.h>
+
+static float el_to_f32(int dtype, const void* p, size_t i)
+{
+    if (dtype == 0) return ((const float*)p)[i];
+    if (dtype == 1) return u2f(orc_f16_to_f32bits(((const uint16_t*)p)[i]));
+    return u2f(orc_bf16_to_f32bits(((const uint16_t*)p)[i]));
+}
+
+/* T(x) * w in T, for one element; x already carries the scale */
+static void store_scaled(int dtype, void* out, size_t i, float xs, const void* w, size_t wi)
+{
+    if (dtype == 0) {
+        float t = xs;                       /* separate statements: no contraction into one rounding */
+        ((float*)out)[i] = t * ((const float*)w)[wi];
+    } else if (dtype == 1) {
+        float t = u2f(orc_f16_to_f32bits(orc_f32bits_to_f16(f2u(xs))));
+        float p = t * u2f(orc_f16_to_f32bits(((const uint16_t*)w)[wi]));     /* exact: 11 + 11 bits fit fp32 */
+        ((uint16_t*)out)[i] = orc_f32bits_to_f16(f2u(p));
+    } else {
+        float t = u2f(orc_bf16_to_f32bits(orc_f32bits_to_bf16(f2u(xs))));
+        float p = t * u2f(orc_bf16_to_f32bits(((const uint16_t*)w)[wi]));    /* exact: 8 + 8 bits */
+        ((uint16_t*)out)[i] = orc_f32bits_to_bf16(f2u(p));
+    }
+}
+
+void orc_norm_geometry(size_t hidden, int dtype, unsigned* vecs, unsigned* vpl, unsigned* lanes)
+{
+    size_t epv = dtype == 0 ? 4 : 8, nv = hidden / epv;
+    unsigned v = (unsigned)((nv + 1023) / 1024);
+    v = v <= 1 ? 1 : v == 2 ? 2 : 4;
+    if (vecs) *vecs = (unsigned)nv;
+    if (vpl) *vpl = v;
+    if (lanes) *lanes = (unsigned)(((nv + v - 1) / v + 63) / 64 * 64);
+}
+
+/* x: rows x hidden elements in storage type `dtype` (already the sum); w: hidden elements. */
+int orc_rmsnorm_rows(int dtype, const void* x, const void* w, void* normed, size_t rows, size_t hidden, float eps)
+{
+    size_t epv = dtype == 0 ? 4 : 8;
+    if (dtype < 0 || dtype > 2 || hidden == 0 || hidden % epv) return -1;
+    unsigned nv, vpl, lanes;
+    orc_norm_geometry(hidden, dtype, &nv, &vpl, &lanes);
+    if (nv > 4096) return -1;
+    float* lane = (float*)malloc(sizeof(float) * lanes);
+    if (!lane) return -1;
+    for (size_t r = 0; r < rows; r++) {
+        const size_t base = r * hidden;
+        for (unsigned t = 0; t < lanes; t++) {
+            float acc = 0.0f;
+            for (unsigned v = 0; v < vpl; v++) {
+                size_t j = (size_t)t + (size_t)v * lanes;
+                if (j >= nv) continue;
+                for (size_t e = 0; e < epv; e++) { float f = el_to_f32(dtype, x, base + j * epv + e); acc = fmaf(f, f, acc); }
+            }
+            lane[t] = acc;
+        }
+        float total = 0.0f;
+        for (unsigned w0 = 0; w0 < lanes; w0 += 64) {
+            float* v = lane + w0;
+            for (unsigned off = 32; off >= 1; off >>= 1) {
+                float nxt[64];
+                for (unsigned i = 0; i < 64; i++) nxt[i] = v[i] + v[i ^ off];
+                memcpy(v, nxt, sizeof nxt);
+            }
+            total = w0 == 0 ? v[0] : total + v[0];
+        }
+        float mean = total / (float)hidden;
+        float var = mean + eps;
+        float s = 1.0f / sqrtf(var);
+        for (size_t i = 0; i < hidden; i++) {
+            float xs = el_to_f32(dtype, x, base + i) * s;
+            store_scaled(dtype, normed, base + i, xs, w, i);
+        }
+    }
+    free(lane);
+    return 0;
+}
+
+/* out = a + b (orc_sum), normed = rmsnorm(out) * w */
+int orc_sum_rmsnorm(int dtype, const void* a, const void* b, const void* w, void* out, void* normed,
+                    size_t rows, size_t hidden, float eps)
+{
+    if (orc_sum(dtype, a, b, out, rows * hidden) != 0) return -1;
+    return orc_rmsnorm_rows(dtype, out, w, normed, rows, hidden, eps);
+}
