@@ -22,6 +22,7 @@ from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also
                    call) and, as decode_latency_stream_gate, the reference's sequence
                    pack kernel, hipStreamWaitValue64, sum kernel
   pipeline_64MiB_fp16  64 MiB fp16 as 16 chunks of 4 MiB over 2 rails x 4 slots
+  sum_rmsnorm_fusion   the sum fused with the following RMSNorm against the two kernels apart
   cpu_baseline     the CPU oracle's restatement of the same step on the host cores.
 """
 import argparse
@@ -247,6 +248,52 @@ def run_pipeline(tbv, torch, synth, st, reps=20):
                     "host clock from the call to the stream's completion, median"}
 
 
+def run_rmsnorm_fusion(tbv, torch, synth, st):
+    """Sum fused with the following RMSNorm (one row kernel: read local and received, write the sum and the
+    normalised row, 4N) against the sum kernel followed by a norm-only launch (3N + 2N), on the prefill shape
+    (cache-cold, 24 rotating buffer sets) and on decode shapes; both orders bit-identical."""
+    lib = tbv.load()
+    hidden = 4096
+    out = {"what": "tbv_emu_run_sum_norm mode 1 (fused, 4N) vs tbv_emu_run_sum + mode 0 (sum 3N, then norm 2N); bf16, hidden 4096; "
+                   "GPU events around 240 launches over 24 rotating buffer sets; us per step"}
+    w = torch.from_numpy(1.0 + 0.25 * synth.normal(5, hidden)).to(torch.bfloat16).cuda()
+    ps = st.cuda_stream
+    for rows in (1, 128, 2048):
+        nset = 24 if rows == 2048 else 4
+        n = rows * hidden * 2
+        A = [torch.from_numpy(synth.normal(10 + i, rows * hidden)).to(torch.bfloat16).cuda() for i in range(2)]
+        sets = [(A[0].clone(), A[1].clone(), torch.empty_like(A[0]), torch.empty_like(A[0])) for _ in range(nset)]
+
+        def fused(i):
+            a, b, o, nm = sets[i % nset]
+            lib.tbv_emu_run_sum_norm(1, o.data_ptr(), a.data_ptr(), b.data_ptr(), nm.data_ptr(), w.data_ptr(), 1e-6, rows, hidden, 2, ps)
+
+        def separate(i):
+            a, b, o, nm = sets[i % nset]
+            lib.tbv_emu_run_sum(o.data_ptr(), a.data_ptr(), b.data_ptr(), n, 2, ps)
+            lib.tbv_emu_run_sum_norm(0, None, o.data_ptr(), None, nm.data_ptr(), w.data_ptr(), 1e-6, rows, hidden, 2, ps)
+
+        res = {}
+        with torch.cuda.stream(st):
+            for name, fn in (("fused", fused), ("separate", separate)):
+                for i in range(nset):
+                    fn(i)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for i in range(240):
+                    fn(i)
+                e1.record()
+                torch.cuda.synchronize()
+                res[name] = e0.elapsed_time(e1) * 1e3 / 240
+            fused(0); torch.cuda.synchronize(); f_out, f_nm = sets[0][2].clone(), sets[0][3].clone()
+            separate(0); torch.cuda.synchronize()
+            same = bool(torch.equal(f_out, sets[0][2])) and bool(torch.equal(f_nm.view(torch.int16), sets[0][3].view(torch.int16)))
+        out[f"rows_{rows}"] = {"fused_us": round(res["fused"], 2), "separate_us": round(res["separate"], 2),
+                               "saved_us": round(res["separate"] - res["fused"], 2), "bit_identical": same,
+                               "fused_GBps_4N": round(4 * n / res["fused"] / 1e3, 1), "fused_frac_of_peak": round(4 * n / (res["fused"] * 1e-6) / HBM_PEAK, 4)}
+    return out
+
+
 def run_cpu_baseline(torch, synth):
     """The oracle's restatement of the same step (memcpy pack + fp32-upcast sum, RNE) on the host cores."""
     from oracle import oracle
@@ -272,7 +319,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
-    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,cpu",
+    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,rmsnorm,cpu",
                     help="comma list of the extra legs to run beside the headline (cold) leg")
     ap.add_argument("--headline-env", default="", help="TBV_X=v,... applied to the headline leg (for profiling one variant)")
     ap.add_argument("--rotate", default=f"{COLD_NSLOT},{COLD_NBUF}",
@@ -381,6 +428,8 @@ def main():
         line["decode_latency_stream_gate"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=False)
     if "pipeline" in legs:
         line["pipeline_64MiB_fp16"] = run_pipeline(tbv, torch, synth, st)
+    if "rmsnorm" in legs:
+        line["sum_rmsnorm_fusion"] = run_rmsnorm_fusion(tbv, torch, synth, st)
     if "cpu" in legs:
         line["cpu_baseline"] = run_cpu_baseline(torch, synth)
     print(json.dumps(line), flush=True)

@@ -8,7 +8,7 @@
 // kernel's result, step4/libtbvcoll.cpp:162-166), x = float(z), s = 1 / sqrt(mean(x^2) + eps),
 // normed = T(x * s) * weight with the product taken in the storage type.
 //
-// One block per row.  Lane t of L holds vectors t, t+L, ... of the row in registers, so the
+// One block per row (L = 64..512 lanes).  Lane t of L holds vectors t, t+L, ... of the row in registers, so the
 // row is read once; the sum of squares is accumulated with fused multiply-adds in a fixed
 // order (per lane: its vectors in order, elements in order; per wave: xor butterfly 32, 16,
 // 8, 4, 2, 1; per block: the waves' totals in wave order), which makes the result
@@ -157,7 +157,8 @@ hipError_t launch_vpl(int vpl, int grid, int block, hipStream_t st, const Timing
     switch (vpl) {
         case 1: return launch2(k_row_norm<DT, 1, MODE>, grid, block, st, t, s, n);
         case 2: return launch2(k_row_norm<DT, 2, MODE>, grid, block, st, t, s, n);
-        default: return launch2(k_row_norm<DT, 4, MODE>, grid, block, st, t, s, n);
+        case 4: return launch2(k_row_norm<DT, 4, MODE>, grid, block, st, t, s, n);
+        default: return launch2(k_row_norm<DT, 8, MODE>, grid, block, st, t, s, n);
     }
 }
 
@@ -199,8 +200,11 @@ hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const 
     s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.a = (const u32x4*)q.a; s.nbytes = q.nbytes; s.seq = q.seq;
-    int vpl = (int)((nm.row_vecs + kMaxSmallThreads - 1) / kMaxSmallThreads);
-    vpl = vpl <= 1 ? 1 : vpl == 2 ? 2 : 4;
+    // Lanes per row: the fewest vectors per lane (1, 2, 4, 8) that bring a row down to 256 lanes, so that eight rows
+    // fit a CU at once.  Measured with 2048 x 4096 bf16, cache-cold: 512 lanes x 1 vector 15.7 us, 256 x 2 14.0 us,
+    // 128 x 4 13.6 us (but 128 decode rows 4.0 us instead of 3.6), 64 x 8 16.0 us.
+    int vpl = 1;
+    while (vpl < 8 && (nm.row_vecs + vpl - 1) / vpl > 256) vpl *= 2;
     int block = (int)(((nm.row_vecs + vpl - 1) / vpl + 63) / 64 * 64);
     const int grid = (int)nm.rows;
     switch (mode) {

@@ -361,7 +361,7 @@ double orc_time_reduce_copy(int dtype, const void* local, const void* peer, void
  * the elements of vectors t, t+L, t+2L, ... in index order; each 64-lane wave is reduced by the
  * xor butterfly 32,16,8,4,2,1; the waves' totals are added in wave order.  1/sqrt is the
  * correctly rounded division of the correctly rounded square root.  L follows from the row:
- * vpl = ceil(vectors / 1024) rounded up to 1, 2 or 4; L = ceil(vectors / vpl) rounded up to 64.
+ * vpl = the smallest of 1, 2, 4, 8 with ceil(vectors / vpl) <= 256 (else 8); L = ceil(vectors / vpl) rounded up to 64.
  * Pinned in the tests against torch's fp32 formula (x.float().pow(2).mean(-1), rsqrt) within 2 ulp
  * of T, and against closed-form rows.
  */
@@ -394,8 +394,8 @@ static void store_scaled(int dtype, void* out, size_t i, float xs, const void* w
 void orc_norm_geometry(size_t hidden, int dtype, unsigned* vecs, unsigned* vpl, unsigned* lanes)
 {
     size_t epv = dtype == 0 ? 4 : 8, nv = hidden / epv;
-    unsigned v = (unsigned)((nv + 1023) / 1024);
-    v = v <= 1 ? 1 : v == 2 ? 2 : 4;
+    unsigned v = 1;
+    while (v < 8 && (nv + v - 1) / v > 256) v *= 2;
     if (vecs) *vecs = (unsigned)nv;
     if (vpl) *vpl = v;
     if (lanes) *lanes = (unsigned)(((nv + v - 1) / v + 63) / 64 * 64);
