@@ -194,6 +194,23 @@ int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, int dtype, vo
 int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, const void* weight, float eps,
                              size_t rows, size_t hidden, int dtype, void* stream);
 
+/* int8 payload codec (TBV_CODEC=1, off by default; payloads of at least TBV_CODEC_MIN bytes,
+ * default 512 KiB, made of whole 16-byte vectors).  The reference plans it as its next feature
+ * and has no code for it (reports/12_references.md:134: bf16 -> int8 blockwise, group 128,
+ * asymmetric; behind a size threshold since it changes the numerics, :140-142).  With the codec
+ * on, tbv_ar_allreduce's pack kernel writes the int8 image of the local tensor into the bounce
+ * slot (groups of 128 elements: scale = (max - min) / 255 and min as fp32, one code byte per
+ * element; 2176 bytes per 2048 elements = 0.53 of a 2-byte payload on the wire) and its sum kernel
+ * writes out = T(decode(own image) + decode(received image)): every rank decodes its own payload
+ * too, so the two ranks of a pair compute the same bits.  |decode(x) - x| <= scale / 2 per
+ * element.  An emulated peer's payload is quantised for it; with tbv_emu_peer_resident it must
+ * have exactly the call's size.
+ * The three functions below run the codec kernels alone, for benches and tests: the image size of
+ * a payload, payload -> image, and two images -> sum. */
+size_t tbv_emu_codec_image_bytes(size_t nbytes, int dtype);
+int tbv_emu_run_quant(void* image, const void* src, size_t nbytes, int dtype, void* stream);
+int tbv_emu_run_sum_quant(void* out, const void* own_image, const void* recv_image, size_t nbytes, int dtype, void* stream);
+
 /* Standalone row kernel for benches and tests: mode 0: normed = rmsnorm(a) * weight;
  * mode 1: out = a + b, normed = rmsnorm(out) * weight. */
 int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const void* b, void* normed, const void* weight, float eps,

@@ -32,7 +32,7 @@ extern "C" int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype,
     hipStream_t st = (hipStream_t)stream;
     note_stream(stream, nbytes);
     const double te = nowt();
-    Call c;
+    Call c{};
     if (enqueue_pack(ptr, outp, nbytes, dtype, st, &c) != 0) return -1;
     if (enqueue_wait_sum(ptr, outp, dtype, st, c) != 0) return -1;
     if (flush_pending() != 0) FAIL("deferred signal launch failed");
@@ -225,6 +225,7 @@ extern "C" int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, in
     const size_t n = (nbytes + chunk - 1) / chunk;
     const size_t depth = std::min<size_t>((size_t)G.nslot - 1, n);
     std::vector<Call> calls(n);
+    for (auto& k : calls) k.out_unaligned = (((uintptr_t)outp) & 15) != 0;    // chunk offsets keep the base's alignment or the codec is off anyway
     auto piece = [&](size_t i, size_t* off, size_t* len) { *off = i * chunk; *len = std::min(chunk, nbytes - *off); };
     const double te = nowt();
     size_t off, len;
@@ -267,7 +268,7 @@ extern "C" int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, con
     note_stream(stream, nbytes);
     NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
     const double te = nowt();
-    Call c;
+    Call c{};
     if (enqueue_pack(ptr, outp, nbytes, dtype, st, &c, &nm) != 0) return -1;
     if (enqueue_wait_sum(ptr, outp, dtype, st, c, &nm) != 0) return -1;
     if (flush_pending() != 0) FAIL("deferred signal launch failed");
@@ -285,6 +286,26 @@ extern "C" int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const vo
     sa.out = out; sa.a = a; sa.b = b; sa.nbytes = rows * hidden * esz; sa.dtype = dtype;
     NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
     return launch_row_norm(mode, nullptr, sa, nm, (hipStream_t)stream) == hipSuccess ? 0 : -1;
+}
+
+// int8 payload codec, standalone for benches and tests (the reference plans the codec, reports/12_references.md:134).
+extern "C" size_t tbv_emu_codec_image_bytes(size_t nbytes, int dtype)
+{
+    return (dtype < 0 || dtype > 2) ? 0 : codec_image_bytes(nbytes, dtype);
+}
+
+extern "C" int tbv_emu_run_quant(void* image, const void* src, size_t nbytes, int dtype, void* stream)
+{
+    PackArgs pa{};
+    pa.dst = image; pa.src = src; pa.nbytes = nbytes; pa.seq = 1;
+    return launch_quant(pa, dtype, (hipStream_t)stream) == hipSuccess ? 0 : -1;
+}
+
+extern "C" int tbv_emu_run_sum_quant(void* out, const void* own_image, const void* recv_image, size_t nbytes, int dtype, void* stream)
+{
+    SumArgs sa{};
+    sa.out = out; sa.a = own_image; sa.b = recv_image; sa.nbytes = nbytes; sa.dtype = dtype;
+    return launch_sum_quant(sa, (hipStream_t)stream) == hipSuccess ? 0 : -1;
 }
 
 extern "C" int tbv_emu_run_pack(const void* src, size_t nbytes, int slot, void* stream)

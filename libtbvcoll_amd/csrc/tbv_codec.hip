@@ -1,0 +1,237 @@
+// int8 payload codec of the all-reduce: the pack kernel quantises the local tensor into the
+// bounce slot (what goes over the wire shrinks to 0.53 of a 2-byte payload), the sum kernel
+// dequantises both ranks' images.
+//
+// The reference plans this as its next feature and has no code for it ("all-reduce payload
+// quantisation, bf16 -> int8 blockwise, group 128, asymmetric", reports/12_references.md:134;
+// it changes the numerics, so it must sit behind a size threshold, :140-142).  Format and
+// arithmetic, all in IEEE fp32 so that a CPU restatement reproduces every byte:
+//
+//   group      128 consecutive elements; mn = min, mx = max of float(x) over the group
+//   scale      (mx - mn) / 255, or 1 when mx == mn;  inv = 255 / (mx - mn), or 0 when mx == mn
+//   code       q = rint((float(x) - mn) * inv) clamped to [0, 255], one byte (mn -> 0, mx -> 255)
+//   decode     r = fma(float(q), scale, mn)
+//   superblock 16 groups: 16 x (scale, mn) as two fp32 each = 128 bytes, then 16 x 128 code bytes
+//              = 2176 bytes for 2048 elements; the image of n elements is ceil(n / 2048)
+//              superblocks (absent elements: code 0, absent groups: scale 0, mn 0)
+//   sum        out = T(decode(own image) + decode(received image)): each rank decodes its OWN
+//              payload too, so both ranks of a pair compute the same bits
+//
+// One lane per 16-byte input vector (8 elements of a 2-byte type, 4 of fp32); the 16 (32) lanes
+// of a group reduce min and max with xor shuffles; one block per superblock per iteration.
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include "tbv_device.h"
+#include "tbv_kernels.h"
+
+namespace tbv {
+
+namespace {
+
+template <int DT> struct Vec;
+template <> struct Vec<0> {
+    static constexpr int EPV = 4;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float* f)
+    {
+        u32x4 r = {__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+        return r;
+    }
+};
+template <> struct Vec<1> {
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        f16x8 h = __builtin_bit_cast(f16x8, v);
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ u32x4 pack(const float* f)
+    {
+        f16x8 h;
+#pragma unroll
+        for (int i = 0; i < 8; i++) h[i] = (_Float16)f[i];
+        return __builtin_bit_cast(u32x4, h);
+    }
+};
+template <> struct Vec<2> {
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ void unpack(u32x4 v, float* f)
+    {
+        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) { f[2 * i] = __uint_as_float(u[i] << 16); f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u); }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float* f)
+    {
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f32x2 s = {f[2 * i], f[2 * i + 1]};
+            bf16x2 r = __builtin_convertvector(s, bf16x2);
+            o[i] = __builtin_bit_cast(uint32_t, r);
+        }
+        u32x4 r = {o[0], o[1], o[2], o[3]};
+        return r;
+    }
+};
+
+static constexpr unsigned kSbHeader = 128;      // 16 x (scale, mn)
+
+template <int DT>
+__global__ __launch_bounds__(512) void k_quant(StepArgs g)
+{
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;             // lanes per group: 16 or 32
+    const unsigned tid = threadIdx.x;                      // blockDim.x = 2048 / EPV: one superblock per iteration
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    const size_t nvec = g.nbytes >> 4;
+    const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
+    unsigned char* image = (unsigned char*)g.bounce;
+    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
+        const size_t i = sb * blockDim.x + tid;
+        const bool have = i < nvec;
+        float f[EPV];
+        float mn = __builtin_inff(), mx = -__builtin_inff();
+        if (have) {
+            Vec<DT>::unpack(g.a[i], f);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+        }
+#pragma unroll
+        for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
+            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+        }
+        const bool group_has = mn <= mx;                       // false when every lane of the group is past the end
+        mn += 0.0f;                                            // a minimum of -0 is stored as +0, whichever zero the reduction met first
+        const float range = mx - mn;
+        const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
+        const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
+        if (!group_has) mn = 0.0f;
+        unsigned char* sbp = image + sb * kCodecSuperBytes;
+        if ((tid % LPG) == 0) {
+            f32x2 hdr = {scale, mn};
+            *(f32x2*)(sbp + (tid / LPG) * 8) = hdr;
+        }
+        uint32_t lo = 0, hi = 0;
+        if (have) {
+#pragma unroll
+            for (int e = 0; e < EPV; e++) {
+                float t = __builtin_rintf((f[e] - mn) * inv);
+                t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
+                const uint32_t q = (uint32_t)t;
+                if (e < 4) lo |= q << (8 * e); else hi |= q << (8 * (e - 4));
+            }
+        }
+        if (EPV == 8) { uint2 c = {lo, hi}; *(uint2*)(sbp + kSbHeader + (size_t)tid * 8) = c; }
+        else *(uint32_t*)(sbp + kSbHeader + (size_t)tid * 4) = lo;
+    }
+    if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
+}
+
+__device__ __forceinline__ void decode(const unsigned char* sbp, unsigned tid, unsigned lpg, int epv, float* r)
+{
+    const f32x2 hdr = *(const f32x2*)(sbp + (tid / lpg) * 8);
+    uint32_t lo, hi = 0;
+    if (epv == 8) { const uint2 c = *(const uint2*)(sbp + kSbHeader + (size_t)tid * 8); lo = c.x; hi = c.y; }
+    else lo = *(const uint32_t*)(sbp + kSbHeader + (size_t)tid * 4);
+    for (int e = 0; e < epv; e++) {
+        const uint32_t q = ((e < 4 ? lo >> (8 * e) : hi >> (8 * (e - 4))) & 0xffu);
+        r[e] = __builtin_fmaf((float)q, hdr.x, hdr.y);
+    }
+}
+
+// out = T(decode(own image) + decode(received image)); g.a = own image, g.b = received image
+template <int DT>
+__global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
+{
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;
+    const unsigned tid = threadIdx.x;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    const size_t nvec = g.nbytes >> 4;
+    const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
+    const unsigned char* ia = (const unsigned char*)g.a;
+    const unsigned char* ib = (const unsigned char*)g.b;
+    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
+        const size_t i = sb * blockDim.x + tid;
+        if (i >= nvec) continue;
+        float x[EPV], y[EPV];
+        decode(ia + sb * kCodecSuperBytes, tid, LPG, EPV, x);
+        decode(ib + sb * kCodecSuperBytes, tid, LPG, EPV, y);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
+        __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + i);
+    }
+    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+}
+
+inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+template <typename A>
+hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const Timing* t, const A& arg)
+{
+    if (t && t->start && t->stop) hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, t->start, t->stop, 0, arg);
+    else hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, arg);
+    return hipGetLastError();
+}
+
+int codec_grid(size_t nbytes, int dtype, bool gated)
+{
+    const size_t epv = dtype == 0 ? 4 : 8, nsb = ((nbytes >> 4) * epv + kCodecSuper - 1) / kCodecSuper;
+    const size_t cap = gated ? 256 : 2048;
+    return (int)(nsb < 1 ? 1 : nsb < cap ? nsb : cap);
+}
+
+}  // namespace
+
+size_t codec_image_bytes(size_t nbytes, int dtype)
+{
+    const size_t esz = dtype == 0 ? 4 : 2, n = nbytes / esz;
+    return (n + kCodecSuper - 1) / kCodecSuper * kCodecSuperBytes;
+}
+
+// Quantise `a.src` (a.nbytes of `dtype`, whole 16-byte vectors) into the image at a.dst; completion signal as the pack's.
+hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timing* t)
+{
+    if (!a.dst || !a.src || (a.cflag && !a.arrive) || !al16(a.dst) || !al16(a.src) || (a.nbytes & 15) || dtype < 0 || dtype > 2 || a.tagp)
+        return hipErrorInvalidValue;
+    StepArgs s{};
+    s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive;
+    s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp; s.sigmode = a.sigmode;
+    s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
+    const int grid = codec_grid(a.nbytes, dtype, false);
+    switch (dtype) {
+        case 0: return launch1(k_quant<0>, grid, 512, st, t, s);
+        case 1: return launch1(k_quant<1>, grid, 256, st, t, s);
+        default: return launch1(k_quant<2>, grid, 256, st, t, s);
+    }
+}
+
+// out = T(decode(q.a) + decode(q.b)) where q.a and q.b are images of q.nbytes of `dtype`.
+hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
+{
+    if (!q.out || !q.a || !q.b || !al16(q.out) || !al16(q.a) || !al16(q.b) || (q.nbytes & 15) || q.dtype < 0 || q.dtype > 2 ||
+        (q.done && !q.done_arrive))
+        return hipErrorInvalidValue;
+    StepArgs s{};
+    s.out = (u32x4*)q.out; s.a = (const u32x4*)q.a; s.b = (const u32x4*)q.b; s.nbytes = q.nbytes; s.seq = q.seq; s.fp = q.fp;
+    s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.done = q.done; s.done_arrive = q.done_arrive;
+    s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
+    const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr);
+    switch (q.dtype) {
+        case 0: return launch1(k_sum_quant<0>, grid, 512, st, t, s);
+        case 1: return launch1(k_sum_quant<1>, grid, 256, st, t, s);
+        default: return launch1(k_sum_quant<2>, grid, 256, st, t, s);
+    }
+}
+
+}  // namespace tbv

@@ -282,6 +282,8 @@ int configure(const char* devs, size_t cap)
     G.R = count_rails(devs);
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
     G.merge = geti("TBV_MERGE", 1);
+    G.codec = geti("TBV_CODEC", 0);
+    G.codec_min = getz("TBV_CODEC_MIN", (size_t)512 << 10);
     // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
     // 256 MB Infinity Cache they stay resident from call to call; beyond that every operand streams from HBM.
     { const size_t working_set = 2 * (size_t)G.nslot * G.stride + 2 * G.cap;
@@ -306,9 +308,15 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
     c->fused = false;
     c->deferred = false;
     c->host_wire = G.async && use_host_wire(st);
+    // The int8 codec applies from a size threshold upwards (below it the wire is a small part of a call), to
+    // whole 16-byte vectors, and not together with the modes that cut or extend the payload on the wire.
+    c->codec = G.codec && G.async && G.gpusig && nbytes >= G.codec_min && !(nbytes & 15) && !G.tag && G.kwait != 1 &&
+               !(G.railsum && c->R > 1) && !nm && !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15) && !c->out_unaligned &&
+               codec_image_bytes(nbytes, dtype) <= G.stride;
+    if (c->codec) c->xbytes = codec_image_bytes(nbytes, dtype);
 
     const char* peer = nullptr;
-    if (peer_assign(c, nbytes, &peer) != 0) return -1;
+    if (peer_assign(c, nbytes, dtype, &peer) != 0) return -1;
 
     PackArgs pa{};
     pa.dst = slot_send(c->slot); pa.src = ptr; pa.nbytes = nbytes;
@@ -323,7 +331,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         if (c->resident) st_rel(gflag(c->slot), c->seq);      // the peer was early: its flag is already up
         if (G.gpusig) {
             const bool aligned = !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
-            const bool plain = sum_out && !G.tag && G.kwait != 1 && !(G.railsum && c->R > 1) && aligned;
+            const bool plain = sum_out && !G.tag && G.kwait != 1 && !(G.railsum && c->R > 1) && aligned && !c->codec;
             const bool can_fuse = G.fuse && c->resident && plain && !nm;
             // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
             // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
@@ -364,7 +372,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             } else {
                 if (c->deferred) pa.cflag = nullptr;
                 KTimer kt(0);
-                if (launch_pack(pa, st, kt.get()) != hipSuccess) FAIL("pack kernel launch failed");
+                if ((c->codec ? launch_quant(pa, dtype, st, kt.get()) : launch_pack(pa, st, kt.get())) != hipSuccess) FAIL("pack kernel launch failed");
                 if (c->deferred) { G.pending.word = cflag(c->slot); G.pending.seq = c->seq; G.pending_stream = st; }
             }
         } else {
@@ -418,7 +426,9 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         KTimer kt(1);
         // with a norm to follow and the whole payload in this piece, the sum kernel is the row kernel that also normalises
         const bool with_norm = nm && off == 0 && len == c.nbytes;
-        if ((with_norm ? launch_row_norm(1, nullptr, sa, *nm, st, kt.get()) : launch_sum(sa, st, kt.get())) != hipSuccess)
+        if (c.codec) sa.a = slot_send(c.slot);               // this rank's own payload as the peer sees it: its image
+        if ((c.codec ? launch_sum_quant(sa, st, kt.get())
+             : with_norm ? launch_row_norm(1, nullptr, sa, *nm, st, kt.get()) : launch_sum(sa, st, kt.get())) != hipSuccess)
             FAIL("sum kernel launch failed");
         return 0;
     };
@@ -548,6 +558,7 @@ int init_impl(int rank, const char* devs, size_t cap)
         x.rl_post = x.rl_arr = 0; x.rl_n = 0;
         if (hipStreamCreateWithFlags(&x.wire, hipStreamNonBlocking) != hipSuccess) FAIL("side stream creation failed");
     }
+    if (G.codec && hipStreamCreateWithFlags(&G.util, hipStreamNonBlocking) != hipSuccess) FAIL("utility stream creation failed");
     for (int i = 0; i < MAXSLOT; i++) { G.rails_done[i].store(0); G.released[i].store(0); G.resident_ok[i] = false; }
     G.caller_napping.store(0);
     for (int r = 0; r < MAXRAIL; r++) G.hold[r].store(0);
@@ -576,6 +587,7 @@ int init_impl(int rank, const char* devs, size_t cap)
     LOGF("  wire %s; copy-engine access for the host wire: %s", G.wire_mode == 1 ? "stream" : G.wire_mode == 2 ? "host" : "auto", dma ? "yes" : "no");
     LOGF("  small calls (<= %zu B) in one kernel: %s", G.fusewait_max, G.onekernel ? "yes" : "no");
     LOGF("  deferred pack signal %s", G.defer ? "on (early peer, or flag polled inside the sum kernel)" : "off");
+    if (G.codec) LOGF("  int8 payload codec for payloads of at least %zu B (group 128, asymmetric, 0.53 of a 2-byte payload on the wire)", G.codec_min);
     LOGF("  cache hints: %s profile; early peer above the one-kernel size: %s", G.streaming ? "streaming" : "resident",
          G.fuse ? "pack+sum fused (4N)" : G.merge ? "pack and sum blocks in one launch" : "two launches");
     return 0;
@@ -601,6 +613,7 @@ void teardown()
     stop_progress();
     for (int r = 0; r < MAXRAIL; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
     peer_teardown();
+    if (G.util) { (void)hipStreamDestroy(G.util); G.util = nullptr; }
     for (int i = 0; i < MAXSLOT; i++) if (G.ev[i]) { (void)hipEventDestroy(G.ev[i]); G.ev[i] = nullptr; }
     if (G.switch_ev) { (void)hipEventDestroy(G.switch_ev); G.switch_ev = nullptr; }
     free_slab(G.sendbase, g_uc_send); G.sendbase = nullptr;

@@ -69,6 +69,8 @@ struct Staged { const char* ptr; size_t nbytes; bool owned; };
 // What enqueue_pack decides about a call and enqueue_wait_sum needs to know.
 struct Call {
     uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused; bool deferred; bool host_wire;
+    bool codec;               // the payload travels as its int8 image (decided by enqueue_pack)
+    bool out_unaligned;       // set by the caller before enqueue_pack when the output is not 16-byte aligned
 };
 
 struct Engine {
@@ -77,6 +79,8 @@ struct Engine {
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     int merge = 1;                            // resident peer: pack and sum blocks in one launch (TBV_MERGE)
     int streaming = 0;                        // cache-hint profile of the large kernels (TBV_STREAMING, default by ring size)
+    int codec = 0;                            // int8 payload codec for payloads of at least codec_min bytes (TBV_CODEC, off by default)
+    size_t codec_min = (size_t)512 << 10;     // TBV_CODEC_MIN
     size_t cap = 0, stride = 0, rail1max = 96u * 1024u, chunkb = 0, fusewait_max = 0;
     double wdog = 10.0;
     double tick_hz = 1e8;                     // rate of the constant clock the kernels bound their waits with
@@ -111,6 +115,8 @@ struct Engine {
     size_t resident_bytes = 0;
     char* resident_src = nullptr;             // device copy of the resident payload, to restore a slot another payload went through
     bool resident_ok[MAXSLOT] = {};           // the receive slot still holds the resident payload
+    int resident_form = -1;                   // what the receive slots hold of it: -1 the raw bytes, else the int8 image for this dtype
+    hipStream_t util = nullptr;               // caller-thread stream for the emulated peer's own preparation work
     int hooks = 0;                            // an arrival script or a withheld signal is set (test hooks, off the default path)
     std::vector<int> script;
     std::atomic<size_t> turn{0};
@@ -204,7 +210,7 @@ int drain_rails();
 // (replaces do_xfer_rail, step4/libtbvcoll.cpp:172-211).  Returns 0, or -1 on error / watchdog.
 int wire_xfer(Rail& x, const Item& it);
 // Whose payload plays the peer for call `c` of `nbytes`: sets *peer (null = mirror) and c->resident.
-int peer_assign(Call* c, size_t nbytes, const char** peer);
+int peer_assign(Call* c, size_t nbytes, int dtype, const char** peer);
 // Must this caller stream's calls be deposited by copy engines rather than a side stream?
 bool use_host_wire(hipStream_t st);
 hipError_t stream_bump(hipStream_t st, unsigned long long* w, uint64_t v);

@@ -98,6 +98,14 @@ bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype);
 // mode 2: the whole small call in one launch (pack `p`, completion word, flag poll, sum, norm).
 hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& s, const NormArgs& n, hipStream_t st, const Timing* t = nullptr);
 
+// int8 payload codec (tbv_codec.hip): groups of 128 elements, 16 groups to a superblock of 2176 bytes.
+static constexpr unsigned kCodecGroup = 128;
+static constexpr unsigned kCodecSuper = 2048;          // elements per superblock
+static constexpr unsigned kCodecSuperBytes = 2176;     // 16 x 8 header bytes + 2048 code bytes
+size_t codec_image_bytes(size_t nbytes, int dtype);
+hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timing* t = nullptr);
+hipError_t launch_sum_quant(const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+
 // Looks up this device's copy of the built-in counter array of tbv_step_noalloc (once per device).
 bool noalloc_bind_device();
 

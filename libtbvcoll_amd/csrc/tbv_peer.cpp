@@ -95,15 +95,17 @@ bool pointer_is_host(const void* p)
     return at.type == hipMemoryTypeHost;
 }
 
-// Device copies of host-staged payloads are released on the caller's thread once no call can read them
-// (the cheap conservative test: nothing is in flight when every rail's queue is empty).
+// Device buffers the emulated peer owns (copies of host-staged payloads, int8 images) are released on the
+// caller's thread once the call that reads them has been released: only the wire reads them, and a call is
+// released after its last rail has seen its fragment arrive.
 void reap_owned()
 {
-    if (G.owned.empty() || !rails_idle()) return;
-    const uint64_t done = G.seq;
+    if (G.owned.empty()) return;
     size_t k = 0;
     for (auto& o : G.owned) {
-        if (o.second && o.second <= done) (void)hipFree(o.first);
+        const bool over = o.second && o.second != ~0ull &&
+                          G.released[(int)(o.second % (uint64_t)G.nslot)].load(std::memory_order_acquire) >= o.second;
+        if (over) (void)hipFree(o.first);
         else G.owned[k++] = o;
     }
     G.owned.resize(k);
@@ -118,6 +120,39 @@ const char* to_device(const void* src, size_t nbytes)
     if (nbytes && hipMemcpy(d, src, nbytes, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(d); return nullptr; }
     G.owned.emplace_back(d, 0);
     return d;
+}
+
+// The int8 image of a peer payload, made the way the peer's own pack kernel would make it (on the caller's
+// thread, on the utility stream, waited for).  The buffer is released once call `seq` is over.
+const char* peer_image(const char* payload, size_t nbytes, int dtype, uint64_t seq)
+{
+    char* img = nullptr;
+    if (hipMalloc((void**)&img, codec_image_bytes(nbytes, dtype)) != hipSuccess) return nullptr;
+    PackArgs pa{};
+    pa.dst = img; pa.src = payload; pa.nbytes = nbytes; pa.seq = seq;
+    if (launch_quant(pa, dtype, G.util) != hipSuccess || hipStreamSynchronize(G.util) != hipSuccess) { (void)hipFree(img); return nullptr; }
+    G.owned.emplace_back(img, seq);
+    return img;
+}
+
+// Put the resident payload into every receive slot in the wanted form: raw (-1) or as its int8 image for `form`.
+int resident_refill(int form)
+{
+    if (drain_rails() != 0) return -1;
+    if (hipDeviceSynchronize() != hipSuccess) return -1;         // no earlier sum may still be reading a slot
+    for (int s = 0; s < G.nslot; s++) {
+        if (form < 0) {
+            if (hipMemcpy(slot_recv(s), G.resident_src, G.resident_bytes, hipMemcpyDeviceToDevice) != hipSuccess) return -1;
+        } else {
+            PackArgs pa{};
+            pa.dst = slot_recv(s); pa.src = G.resident_src; pa.nbytes = G.resident_bytes;
+            if (!G.util || launch_quant(pa, form, G.util) != hipSuccess) return -1;
+        }
+        G.resident_ok[s] = true;
+    }
+    if (form >= 0 && hipStreamSynchronize(G.util) != hipSuccess) return -1;
+    G.resident_form = form;
+    return 0;
 }
 
 void refresh_hooks()
@@ -244,26 +279,38 @@ bool use_host_wire(hipStream_t st)
 // Whose payload plays the peer for this call: a staged one (FIFO), the resident one (already in the
 // receive slot, or put back through the wire when another payload went through that slot since),
 // the repeat payload, or none (mirror: the peer echoes this rank's bounce slot).
-int peer_assign(Call* c, size_t nbytes, const char** peer)
+int peer_assign(Call* c, size_t nbytes, int dtype, const char** peer)
 {
     *peer = nullptr;
     c->resident = false;
+    bool from_resident = false;
     if (!G.staged.empty()) {
         Staged s = G.staged.front(); G.staged.pop_front();
         if (s.nbytes < nbytes) FAIL("staged peer payload (%zu B) is shorter than the call (%zu B)", s.nbytes, nbytes);
         *peer = s.ptr;
         if (s.owned) for (auto& o : G.owned) if (o.first == s.ptr) o.second = c->seq;
     } else if (G.resident_bytes && G.resident_bytes >= nbytes) {
+        // the receive slots hold either the raw payload or its int8 image for one dtype and exactly its size
+        const int form = c->codec ? dtype : -1;
+        if (c->codec && G.resident_bytes != nbytes) FAIL("with the int8 codec an early peer's payload must have the call's size (%zu B, call %zu B)", G.resident_bytes, nbytes);
+        if (form != G.resident_form && resident_refill(form) != 0) return -1;
         if (G.resident_ok[c->slot]) c->resident = true;
-        else *peer = G.resident_src;
+        else { *peer = G.resident_src; from_resident = true; }
     } else if (G.repeat.ptr) {
         if (G.repeat.nbytes < nbytes) FAIL("repeat peer payload (%zu B) is shorter than the call (%zu B)", G.repeat.nbytes, nbytes);
         *peer = G.repeat.ptr;
     }
+    // With the codec the peer's pack kernel would have quantised its payload: do that for it now.
+    if (c->codec && *peer) {
+        reap_owned();
+        const char* img = peer_image(*peer, nbytes, dtype, c->seq);
+        if (!img) FAIL("could not quantise the peer's payload");
+        *peer = img;
+    }
     // Any call that deposits into its slot replaces the resident image there; the image counts as restored
     // only when the resident payload itself went through the wire in full.
     if (G.resident_bytes && !c->resident)
-        G.resident_ok[c->slot] = (*peer == G.resident_src && nbytes >= G.resident_bytes);
+        G.resident_ok[c->slot] = (from_resident && nbytes >= G.resident_bytes);
     return 0;
 }
 
@@ -327,6 +374,7 @@ extern "C" int tbv_emu_peer_resident(const void* src, size_t nbytes)
         G.resident_ok[s] = true;
     }
     G.resident_bytes = nbytes;
+    G.resident_form = -1;
     return 0;
 }
 

@@ -57,6 +57,8 @@ _SIGNATURES = {
     "tbv_emu_hbm_probe": (_I, [_I, _SZ, _SZ, _I, _PD, _PD]), "tbv_emu_launch_floor": (_I, [_I, _PD]),
     "tbv_ar_allreduce_rmsnorm": (_I, [_VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
     "tbv_emu_run_sum_norm": (_I, [_I, _VP, _VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
+    "tbv_emu_codec_image_bytes": (_SZ, [_SZ, _I]),
+    "tbv_emu_run_quant": (_I, [_VP, _VP, _SZ, _I, _VP]), "tbv_emu_run_sum_quant": (_I, [_VP, _VP, _VP, _SZ, _I, _VP]),
 }
 
 

@@ -59,6 +59,10 @@ def lib():
         l.orc_ring_model2.restype = ctypes.c_long
         l.orc_rmsnorm_rows.argtypes = [ci, vp, vp, vp, sz, sz, ctypes.c_float]; l.orc_rmsnorm_rows.restype = ci
         l.orc_sum_rmsnorm.argtypes = [ci, vp, vp, vp, vp, vp, sz, sz, ctypes.c_float]; l.orc_sum_rmsnorm.restype = ci
+        l.orc_q8_image_bytes.argtypes = [sz]; l.orc_q8_image_bytes.restype = sz
+        l.orc_q8_encode.argtypes = [ci, vp, sz, vp]; l.orc_q8_encode.restype = ci
+        l.orc_q8_decode.argtypes = [vp, sz, vp]; l.orc_q8_decode.restype = None
+        l.orc_q8_sum.argtypes = [ci, vp, vp, sz, vp]; l.orc_q8_sum.restype = ci
         l.orc_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci]; l.orc_reduce_copy.restype = ci
         l.orc_time_reduce_copy.argtypes = [ci, vp, vp, vp, vp, sz, ci, ci, ci]; l.orc_time_reduce_copy.restype = ctypes.c_double
         _lib = l
@@ -155,6 +159,27 @@ def sum_rmsnorm(dtype, a, b, w, hidden, eps):
     rc = lib().orc_sum_rmsnorm(dtype, _p(a), _p(b), _p(w), _p(out), _p(normed), a.size // hidden, hidden, eps)
     assert rc == 0
     return out, normed
+
+
+def q8_encode(dtype, x):
+    """int8 codec image (uint8 array) of the storage-bit array x."""
+    x = np.ascontiguousarray(x, dtype=_NP[dtype]).reshape(-1)
+    img = np.zeros(int(lib().orc_q8_image_bytes(x.size)), dtype=np.uint8)
+    assert lib().orc_q8_encode(dtype, _p(x), x.size, _p(img)) == 0
+    return img
+
+
+def q8_decode(img, n):
+    out = np.empty(n, dtype=np.float32)
+    lib().orc_q8_decode(_p(np.ascontiguousarray(img, dtype=np.uint8)), n, _p(out))
+    return out
+
+
+def q8_sum(dtype, own_img, recv_img, n):
+    """out = T(decode(own) + decode(received)) as storage bits."""
+    out = np.empty(n, dtype=_NP[dtype])
+    assert lib().orc_q8_sum(dtype, _p(np.ascontiguousarray(own_img, dtype=np.uint8)), _p(np.ascontiguousarray(recv_img, dtype=np.uint8)), n, _p(out)) == 0
+    return out
 
 
 def reduce_copy(dtype, local, peer, nthreads=1):

@@ -451,3 +451,75 @@ int orc_sum_rmsnorm(int dtype, const void* a, const void* b, const void* w, void
     if (orc_sum(dtype, a, b, out, rows * hidden) != 0) return -1;
     return orc_rmsnorm_rows(dtype, out, w, normed, rows, hidden, eps);
 }
+
+/* ---------------------------------------------------------------- int8 payload codec
+ * Planned in the reference as its next feature, without code ("bf16 -> int8 blockwise, group 128,
+ * asymmetric", reports/12_references.md:134; behind a size threshold because it changes the
+ * numerics, :140-142).  The format restated here is this build's own, stated in IEEE fp32 so that
+ * every byte is reproducible:
+ *   group      128 consecutive elements; mn, mx = min, max of float(x) over the elements present
+ *   scale      (mx - mn) / 255, or 1 when mx == mn;  inv = 255 / (mx - mn), or 0 when mx == mn
+ *   code       q = rint((float(x) - mn) * inv) clamped to [0, 255]   (round half to even)
+ *   decode     r = fma(float(q), scale, mn)
+ *   superblock 16 x (scale, mn) as fp32 pairs, then 16 x 128 code bytes = 2176 bytes per 2048 elements;
+ *              absent elements have code 0, absent groups scale 0 and mn 0
+ *   sum        out = T(decode(own image) + decode(received image))
+ * Pinned in the tests by invariants (|decode - x| <= scale/2, constant group exact, mn -> 0 and
+ * mx -> 255, monotone codes), by an independent float64 numpy computation of the codes (equal
+ * except at rounding boundaries) and by hand-made tiny groups.
+ * Parity unpinned: non-finite inputs.
+ */
+size_t orc_q8_image_bytes(size_t n) { return (n + 2047) / 2048 * 2176; }
+
+int orc_q8_encode(int dtype, const void* src, size_t n, unsigned char* image)
+{
+    if (dtype < 0 || dtype > 2) return -1;
+    memset(image, 0, orc_q8_image_bytes(n));
+    for (size_t g0 = 0; g0 < n; g0 += 128) {
+        size_t cnt = n - g0 < 128 ? n - g0 : 128;
+        float mn = el_to_f32(dtype, src, g0), mx = mn;
+        for (size_t i = 1; i < cnt; i++) { float f = el_to_f32(dtype, src, g0 + i); mn = fminf(mn, f); mx = fmaxf(mx, f); }
+        mn += 0.0f;                                /* a minimum of -0 is stored as +0 */
+        float range = mx - mn;
+        float scale = range > 0.0f ? range / 255.0f : 1.0f;
+        float inv = range > 0.0f ? 255.0f / range : 0.0f;
+        unsigned char* sb = image + (g0 / 2048) * 2176;
+        size_t gi = (g0 % 2048) / 128;
+        memcpy(sb + gi * 8, &scale, 4); memcpy(sb + gi * 8 + 4, &mn, 4);
+        for (size_t i = 0; i < cnt; i++) {
+            float d = el_to_f32(dtype, src, g0 + i) - mn;
+            float t = rintf(d * inv);
+            if (t < 0.0f) t = 0.0f;
+            if (t > 255.0f) t = 255.0f;
+            sb[128 + gi * 128 + i] = (unsigned char)t;
+        }
+    }
+    return 0;
+}
+
+static float q8_decode1(const unsigned char* image, size_t i)
+{
+    const unsigned char* sb = image + (i / 2048) * 2176;
+    size_t gi = (i % 2048) / 128;
+    float scale, mn;
+    memcpy(&scale, sb + gi * 8, 4); memcpy(&mn, sb + gi * 8 + 4, 4);
+    return fmaf((float)sb[128 + (i % 2048)], scale, mn);
+}
+
+void orc_q8_decode(const unsigned char* image, size_t n, float* out)
+{
+    for (size_t i = 0; i < n; i++) out[i] = q8_decode1(image, i);
+}
+
+int orc_q8_sum(int dtype, const unsigned char* own, const unsigned char* recv, size_t n, void* out)
+{
+    if (dtype < 0 || dtype > 2) return -1;
+    for (size_t i = 0; i < n; i++) {
+        float x = q8_decode1(own, i), y = q8_decode1(recv, i);
+        float s = x + y;
+        if (dtype == 0) ((float*)out)[i] = s;
+        else if (dtype == 1) ((uint16_t*)out)[i] = orc_f32bits_to_f16(f2u(s));
+        else ((uint16_t*)out)[i] = orc_f32bits_to_bf16(f2u(s));
+    }
+    return 0;
+}
