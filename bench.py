@@ -22,6 +22,7 @@ from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also
                    call) and, as decode_latency_stream_gate, the reference's sequence
                    pack kernel, hipStreamWaitValue64, sum kernel
   pipeline_64MiB_fp16  64 MiB fp16 as 16 chunks of 4 MiB over 2 rails x 4 slots
+  cold_int8_codec      the cold step with the int8 payload codec on
   sum_rmsnorm_fusion   the sum fused with the following RMSNorm against the two kernels apart
   cpu_baseline     the CPU oracle's restatement of the same step on the host cores.
 """
@@ -41,7 +42,7 @@ N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
 COLD_NSLOT, COLD_NBUF = 16, 12         # 2 x 16 x 16 MiB of rings + 2 x 12 x 16 MiB of tensors = 896 MiB
 TRAFFIC_FILE = os.path.join("profiles", "prefill16MiB_cold_pmc_fetch_write.txt")
-TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL")
+TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL", "TBV_CODEC", "TBV_CODEC_MIN")
 
 
 def pct(xs, q):
@@ -69,7 +70,7 @@ def own_warmup(warmup, nslot, nbuf):
     return max(warmup, 2 * math.lcm(nslot, nbuf), 48)
 
 
-def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0):
+def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0, check="exact"):
     """`steps` timed calls after `warmup` untimed ones (never fewer than two turns of every rotating tensor and
     ring slot, so no buffer is touched for the first time inside the clock), then an optional long run, then a
     pass of the same steps with the dispatch timestamps of every kernel launch."""
@@ -123,7 +124,17 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     torch.cuda.synchronize()           # the averages are per completed transfer: let all of them complete
     enq = tbv.stats4()[3]
     want = a + b
-    ok = all(bool(torch.equal(o, want)) for o in outs)    # the timed path computed the sum, bit for bit
+    if check == "codec":
+        # with the int8 codec every element is within half a quantisation step of each operand's group of 128
+        # (step = (max - min) / 255), plus the rounding of the result to bf16
+        def step_of(t):
+            g = t.float().reshape(-1, 128)
+            return ((g.amax(1) - g.amin(1)) / 255.0).repeat_interleave(128)
+        steps2 = step_of(a) + step_of(b)
+        bound = steps2 * 0.5005 + ((a.float() + b.float()).abs() + steps2) * 2.0 ** -8 + 1e-12
+        ok = all(bool(((o.float() - (a.float() + b.float())).abs() <= bound).all()) for o in outs)
+    else:
+        ok = all(bool(torch.equal(o, want)) for o in outs)    # the timed path computed the sum, bit for bit
     tbv.stats4()
 
     ksteps = max(min(steps, 1000), 240)
@@ -319,7 +330,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
-    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,rmsnorm,cpu",
+    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,codec,rmsnorm,cpu",
                     help="comma list of the extra legs to run beside the headline (cold) leg")
     ap.add_argument("--headline-env", default="", help="TBV_X=v,... applied to the headline leg (for profiling one variant)")
     ap.add_argument("--rotate", default=f"{COLD_NSLOT},{COLD_NBUF}",
@@ -428,6 +439,16 @@ def main():
         line["decode_latency_stream_gate"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=False)
     if "pipeline" in legs:
         line["pipeline_64MiB_fp16"] = run_pipeline(tbv, torch, synth, st)
+    if "codec" in legs:
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, env=(("TBV_CODEC", 1),), check="codec")
+        rms = r["wall"] / sub_steps * 1e3
+        img = 2176 * ((n // 2 + 2047) // 2048)
+        line["cold_int8_codec"] = {"what": "the same cache-cold step with the int8 payload codec (TBV_CODEC=1; group 128, asymmetric): the pack "
+                                           "kernel writes the image of the local tensor, the sum kernel decodes both images; off by default",
+                                   "steps": sub_steps, "ms_per_step": round(rms, 5), "wire_bytes": img, "wire_fraction_of_payload": round(img / n, 4),
+                                   "result_within_half_step_of_each_operand": r["ok"],
+                                   "pack": kernel_roofline(n + img, r["pack_us"], r["pack_min_us"], r["n_pack"], ceiling),
+                                   "sum": kernel_roofline(n + 2 * img, r["sum_us"], r["sum_min_us"], r["n_sum"], ceiling)}
     if "rmsnorm" in legs:
         line["sum_rmsnorm_fusion"] = run_rmsnorm_fusion(tbv, torch, synth, st)
     if "cpu" in legs:

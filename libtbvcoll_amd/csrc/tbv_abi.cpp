@@ -234,12 +234,16 @@ extern "C" int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, in
         if (enqueue_pack((const char*)ptr + off, nullptr, len, dtype, st, &calls[i]) != 0) return -1;
     }
     for (size_t i = 0; i < n; i++) {
-        piece(i, &off, &len);
-        if (enqueue_wait_sum((const char*)ptr + off, (char*)outp + off, dtype, st, calls[i]) != 0) return -1;
+        // the pack of chunk i+depth shares a launch with the sum of chunk i wherever the mode allows
+        PackArgs held{};
+        bool have_held = false;
         if (i + depth < n) {
             piece(i + depth, &off, &len);
-            if (enqueue_pack((const char*)ptr + off, nullptr, len, dtype, st, &calls[i + depth]) != 0) return -1;
+            if (enqueue_pack((const char*)ptr + off, nullptr, len, dtype, st, &calls[i + depth], nullptr, &held) != 0) return -1;
+            have_held = calls[i + depth].held;
         }
+        piece(i, &off, &len);
+        if (enqueue_wait_sum((const char*)ptr + off, (char*)outp + off, dtype, st, calls[i], nullptr, have_held ? &held : nullptr) != 0) return -1;
     }
     if (flush_pending() != 0) FAIL("deferred signal launch failed");
     G.t_enq += nowt() - te;

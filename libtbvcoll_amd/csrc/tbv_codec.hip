@@ -155,7 +155,7 @@ __global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
     constexpr unsigned LPG = kCodecGroup / EPV;
     const unsigned tid = threadIdx.x;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
-    if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+    if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     const size_t nvec = g.nbytes >> 4;
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
     const unsigned char* ia = (const unsigned char*)g.a;
@@ -223,7 +223,7 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
         return hipErrorInvalidValue;
     StepArgs s{};
     s.out = (u32x4*)q.out; s.a = (const u32x4*)q.a; s.b = (const u32x4*)q.b; s.nbytes = q.nbytes; s.seq = q.seq; s.fp = q.fp;
-    s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks; s.b_uncached = q.b_uncached;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
     const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr);

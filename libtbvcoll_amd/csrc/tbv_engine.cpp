@@ -80,6 +80,38 @@ void release_gpu(const Item& it)
 }
 
 // ---- progress thread, one per rail (replaces progress_rail, step4/libtbvcoll.cpp:226-277) ----
+
+// The pack's completion word of one item (every rail watches the same one), bounded by the watchdog counted
+// from `since`.  Returns 1 when it is up, 0 when not yet, -1 when the watchdog has run out (error flag set).
+int pack_complete(const Rail& x, const Item& it, double since, int NS)
+{
+    if (ld_acq(cflag(it.slot)) >= it.seq) return 1;
+    if (nowt() - since <= G.wdog) return 0;
+    unsigned long long* fp = footprints();
+    LOGF("watchdog: rail%d pack completion word not seen for %.0fs seq=%llu", x.idx, G.wdog, (unsigned long long)it.seq);
+    LOGF("  GPU footprints wait-in=%llu wait-out=%llu pack=%llu sum-done=%llu wait-timeout=%llu host-seq=%llu cflag=%llu gflag[prev]=%llu",
+         fp[0], fp[1], fp[2], fp[3], fp[4], (unsigned long long)G.seq, *cflag(it.slot), *gflag((int)((it.seq - 1) % NS)));
+    G.err.store(1);
+    return -1;
+}
+
+// An item is over for this rail: its own flag (per-rail sums start on their own arrival; raised on error too),
+// the GPU's flag when this was the call's last rail (error or not; the counter is put back to 0 by that rail
+// itself), and the queue slot back to the caller.
+void finish_item(Rail& x, const Item& it, uint64_t tail)
+{
+    st_rel(rflag(x.idx, it.slot), it.seq);
+    if (G.rails_done[it.slot].fetch_add(1u, std::memory_order_acq_rel) + 1u >= (unsigned)it.R) release_gpu(it);
+    x.q_tail.store(tail + 1, std::memory_order_seq_cst);
+    wake_if(G.caller_napping, &G.cv_room);
+}
+
+// Two ways through the queue.  The default keeps several transfers in flight, as a NIC with several work
+// requests posted does: every queued item whose pack is complete gets its deposit and arrival signal posted at
+// once (posting does not wait), and items are finished in order as their arrival words come up; sixteen
+// 4 MiB chunks then cost one posting each (5-6 us) instead of posting plus arrival (12 us) one after the other.
+// One item at a time, post then wait (the reference's do_xfer_rail, step4/libtbvcoll.cpp:172-211), remains for
+// the copy-engine wire, whose copies block, for event signalling, and whenever a test hook is set.
 void* progress_rail(void* arg)
 {
     Rail& x = *(Rail*)arg;
@@ -89,6 +121,10 @@ void* progress_rail(void* arg)
         if (pthread_setaffinity_np(pthread_self(), sizeof cs, &cs)) LOGF("rail%d: could not pin to cpu %d", x.idx, G.cpu + x.idx);
     }
     const int NS = G.nslot;
+    uint64_t posted = 0;                        // items [q_tail, posted) have their transfer in flight
+    double t_watch = 0;                         // since when the item at `posted` has been waiting for its pack
+    double t_post0[MAXSLOT], t_post1[MAXSLOT];  // per queue position: posting started / returned
+    bool owns[MAXSLOT];
     while (G.run.load(std::memory_order_acquire)) {
         if (queue_empty(x)) {
             const double ts = nowt();
@@ -104,34 +140,56 @@ void* progress_rail(void* arg)
             if (queue_empty(x)) continue;
         }
         const uint64_t tail = x.q_tail.load(std::memory_order_relaxed);
-        const Item it = x.q[tail % NS];
+        const uint64_t head = x.q_head.load(std::memory_order_acquire);
+        if (posted < tail) { posted = tail; t_watch = 0; }
 
-        // the pack's completion word: every rail watches the same one
-        if (G.gpusig) {
-            const double tw = nowt();
-            while (ld_acq(cflag(it.slot)) < it.seq) {
-                if (nowt() - tw > G.wdog) {
-                    unsigned long long* fp = footprints();
-                    LOGF("watchdog: rail%d pack completion word not seen for %.0fs seq=%llu", x.idx, G.wdog, (unsigned long long)it.seq);
-                    LOGF("  GPU footprints wait-in=%llu wait-out=%llu pack=%llu sum-done=%llu wait-timeout=%llu host-seq=%llu cflag=%llu gflag[prev]=%llu",
-                         fp[0], fp[1], fp[2], fp[3], fp[4], (unsigned long long)G.seq, *cflag(it.slot),
-                         *gflag((int)((it.seq - 1) % NS)));
-                    G.err.store(1);
-                    break;
-                }
+        const Item& oldest = x.q[tail % NS];
+        const bool one_at_a_time = G.hooks || !G.gpusig || oldest.host_wire || G.err.load(std::memory_order_relaxed);
+        if (one_at_a_time && posted == tail) {
+            const Item it = oldest;
+            if (G.gpusig) {
+                const double tw = nowt();
+                int pc;
+                while ((pc = pack_complete(x, it, tw, NS)) == 0) { }
+                const double w = nowt() - tw;
+                if (w > 1.0 && x.idx == 0) LOGF("pack completion word took %.1fs seq=%llu", w, (unsigned long long)it.seq);
+            } else if (hipEventSynchronize(G.ev[it.slot]) != hipSuccess) {
+                G.err.store(1);
             }
-            const double w = nowt() - tw;
-            if (w > 1.0 && x.idx == 0) LOGF("pack completion word took %.1fs seq=%llu", w, (unsigned long long)it.seq);
-        } else if (hipEventSynchronize(G.ev[it.slot]) != hipSuccess) {
-            G.err.store(1);
+            if (!G.err.load() && wire_xfer(x, it) != 0) G.err.store(1);
+            finish_item(x, it, tail);
+            posted = tail + 1; t_watch = 0;
+            continue;
         }
-        if (!G.err.load() && wire_xfer(x, it) != 0) G.err.store(1);
-        // this rail's own flag (per-rail sums start on their own arrival); raised on error too
-        st_rel(rflag(x.idx, it.slot), it.seq);
-        // the last rail to finish releases the GPU, error or not, and puts the counter back to 0 itself
-        if (G.rails_done[it.slot].fetch_add(1u, std::memory_order_acq_rel) + 1u >= (unsigned)it.R) release_gpu(it);
-        x.q_tail.store(tail + 1, std::memory_order_seq_cst);
-        wake_if(G.caller_napping, &G.cv_room);
+
+        // post whatever is ready, in order
+        while (posted < head && !G.err.load(std::memory_order_relaxed)) {
+            const Item& it = x.q[posted % NS];
+            if (it.host_wire || G.hooks) break;                      // that one goes one at a time, once it is the oldest
+            if (t_watch == 0) t_watch = nowt();
+            if (pack_complete(x, it, t_watch, NS) != 1) break;
+            const int k = (int)(posted % NS);
+            t_post0[k] = nowt();
+            if (wire_post(x, it, &owns[k]) != 0) { G.err.store(1); break; }
+            t_post1[k] = nowt();
+            posted++; t_watch = 0;
+        }
+        // finish the oldest one when its fragment has arrived
+        if (posted > tail) {
+            const Item it = oldest;
+            const int k = (int)(tail % NS);
+            bool over = !owns[k] || wire_arrived(x, it);
+            if (!over && nowt() - t_post0[k] > G.wdog) {
+                LOGF("watchdog: rail%d transfer exceeded %.1fs seq=%llu", x.idx, nowt() - t_post0[k], (unsigned long long)it.seq);
+                G.err.store(1);
+            }
+            if (over || G.err.load(std::memory_order_relaxed)) {
+                if (over && owns[k]) wire_done(x, it, t_post0[k], t_post1[k]);
+                finish_item(x, it, tail);
+            }
+        } else if (G.err.load(std::memory_order_relaxed) && posted == tail && tail < head) {
+            continue;                                                // the error path above takes it from here
+        }
     }
     return nullptr;
 }
@@ -265,7 +323,9 @@ int configure(const char* devs, size_t cap)
     G.cpu = geti("TBV_CPU", -1);
     { const char* e = getenv("TBV_WDOG"); G.wdog = (e && atof(e) > 0) ? atof(e) : 10.0; }
     G.tag = (geti("TBV_TAG", 0) && G.async && G.gpusig) ? 1 : 0;
-    G.uncached = geti("TBV_UNCACHED", 1);
+    // bit 0: send ring uncached (the reference's default, step4/libtbvcoll.cpp:314); bit 1: receive ring uncached, the
+    // kind of memory a peer's writes land in (costs the sum nothing: 12.9 us per 16 MiB step either way)
+    G.uncached = geti("TBV_UNCACHED", 3);
     G.railsum = geti("TBV_RAILSUM", 0);
     G.fuse = geti("TBV_FUSE", 0);
     // uncached bounce: waves only drain their stores; cached bounce: block leader writes the L2 back
@@ -297,7 +357,7 @@ int configure(const char* devs, size_t cap)
 
 // First half of a call: sequence number, slot, pack kernel, work items.
 // `sum_out`/`dtype` are only used when the sum can share the pack's launch.
-int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm)
+int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm, PackArgs* hold)
 {
     const size_t tagoff = tag_offset(nbytes);
     c->nbytes = nbytes;
@@ -356,7 +416,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (launch_pack(pa, st) != hipSuccess) FAIL("pack kernel launch failed");
             } else if (one_kernel || can_fuse || can_merge) {
                 SumArgs sa{};
-                sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
+                sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.b_uncached = (G.uncached & 2) != 0; sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 if (one_kernel && !c->resident) {
                     sa.wait_flag = gflag(c->slot); sa.relay = relay_word(c->slot);
                     sa.spin_limit_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);
@@ -369,6 +429,11 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (e != hipSuccess) FAIL("%s launch failed", one_kernel ? "one-kernel call" : "pack+sum kernel");
                 G.t_post += nowt() - tq;                       // the launch that carries the sum
                 c->fused = true;
+            } else if (hold && !c->codec && G.packsig == 0 && !G.tag && G.kwait != 1 && !(((uintptr_t)ptr) & 15)) {
+                // the chunked pipeline launches this pack together with an earlier chunk's sum: hand the arguments back
+                c->deferred = false;
+                c->held = true;
+                *hold = pa;
             } else {
                 if (c->deferred) pa.cflag = nullptr;
                 KTimer kt(0);
@@ -407,9 +472,20 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
 }
 
 // Second half: gate the stream on the flag(s), then the sum.
-int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm)
+// `with_pack`: a later chunk's pack that enqueue_pack handed back, to be launched with this sum (or before it,
+// where the two cannot share a launch).
+int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm, const PackArgs* with_pack)
 {
     if (c.fused) return 0;
+    const bool railsum_path = G.async && G.railsum && c.R > 1 && !G.tag;
+    const bool pipe = with_pack && !railsum_path && !c.codec && !nm && !G.tag && G.kwait != 1 && G.async && G.can_wait_value &&
+                      !(((uintptr_t)ptr | (uintptr_t)outp) & 15);
+    if (with_pack && !pipe) {
+        PackArgs pa = *with_pack;
+        if (!pa.pre.word) pa.pre = take_pending(st);
+        KTimer kt(0);
+        if (launch_pack(pa, st, kt.get()) != hipSuccess) FAIL("pack kernel launch failed");
+    }
     const char* rb = slot_recv(c.slot);
     const unsigned long long spin_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);
     const bool probe = G.probe.load(std::memory_order_relaxed) != 0;
@@ -417,7 +493,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
 
     auto sum_piece = [&](size_t off, size_t len, const unsigned long long* gate, bool last) -> int {
         SumArgs sa{};
-        sa.out = (char*)outp + off; sa.a = (const char*)ptr + off; sa.b = rb + off;
+        sa.out = (char*)outp + off; sa.a = (const char*)ptr + off; sa.b = rb + off; sa.b_uncached = (G.uncached & 2) != 0;
         sa.nbytes = len; sa.dtype = dtype; sa.seq = c.seq;
         sa.wait_flag = gate; sa.relay = gate ? relay_word(c.slot) : nullptr; sa.spin_limit_ticks = spin_ticks;
         sa.fp = G.kwait ? footprints() : nullptr;
@@ -427,6 +503,14 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         // with a norm to follow and the whole payload in this piece, the sum kernel is the row kernel that also normalises
         const bool with_norm = nm && off == 0 && len == c.nbytes;
         if (c.codec) sa.a = slot_send(c.slot);               // this rank's own payload as the peer sees it: its image
+        if (pipe) {
+            PackArgs pa = *with_pack;
+            if (!pa.pre.word) pa.pre = sa.pre;               // at most one signal is pending at a time: the held pack may hold it already
+            sa.pre = PreSignal{};
+            if (gate) { sa.wait_flag = gate; sa.relay = relay_word(c.slot); }
+            if (launch_pipe(pa, sa, st, kt.get()) != hipSuccess) FAIL("pipeline kernel launch failed");
+            return 0;
+        }
         if ((c.codec ? launch_sum_quant(sa, st, kt.get())
              : with_norm ? launch_row_norm(1, nullptr, sa, *nm, st, kt.get()) : launch_sum(sa, st, kt.get())) != hipSuccess)
             FAIL("sum kernel launch failed");
@@ -466,7 +550,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         // place before the sum is even launched and the stream needs no gate at all.
         const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
         // (a row kernel has one block per row and no grid cap: it may only wait inside when its rows are few)
-        const bool fusewait = G.async && !arrived && (c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
+        const bool fusewait = G.async && !arrived && (pipe || c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
                               !(nm && nm->rows > (unsigned)kRowNormMaxSmallRows);
         if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
@@ -543,7 +627,8 @@ int init_impl(int rank, const char* devs, size_t cap)
     const size_t wbytes = (size_t)W_BLOCKS * MAXSLOT * FLAG_STRIDE;
     if (hipHostMalloc((void**)&G.hostwords, wbytes, hipHostMallocCoherent) != hipSuccess) FAIL("host flag block allocation failed");
     memset(G.hostwords, 0, wbytes);
-    const size_t cbytes = sizeof(unsigned int) * 2 * MAXSLOT * kCounterWords + (size_t)MAXSLOT * 64;
+    // [2 x MAXSLOT counter blocks][one block's worth of relay words][MAXRAIL x MAXSLOT counter blocks]
+    const size_t cbytes = sizeof(unsigned int) * ((size_t)2 * MAXSLOT + 1 + (size_t)MAXRAIL * MAXSLOT) * kCounterWords;
     if (hipMalloc((void**)&G.counters, cbytes) != hipSuccess) FAIL("counter allocation failed");
     if (hipMemset(G.counters, 0, cbytes) != hipSuccess) FAIL("counter clear failed");
     for (int i = 0; i < G.nslot; i++) {

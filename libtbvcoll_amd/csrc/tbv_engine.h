@@ -71,6 +71,7 @@ struct Call {
     uint64_t seq; int slot; int R; size_t nbytes, xbytes; bool resident; bool fused; bool deferred; bool host_wire;
     bool codec;               // the payload travels as its int8 image (decided by enqueue_pack)
     bool out_unaligned;       // set by the caller before enqueue_pack when the output is not 16-byte aligned
+    bool held;                // enqueue_pack handed the pack's arguments back instead of launching it
 };
 
 struct Engine {
@@ -89,7 +90,8 @@ struct Engine {
     char* sendbase = nullptr;
     char* recvbase = nullptr;
     char* hostwords = nullptr;                // one coherent host block holding every flag word
-    unsigned int* counters = nullptr;         // device: per slot one counter block for the pack, one for the sum
+    unsigned int* counters = nullptr;         // device: per slot a counter block for the pack and one for the sum, the relay words,
+                                              // and a counter block per (rail, slot) for the emulated peer's deposit kernel
     hipEvent_t ev[MAXSLOT] = {};
     // protocol state
     Rail rr[MAXRAIL];
@@ -173,6 +175,7 @@ inline void st_rel(unsigned long long* p, uint64_t v) { __atomic_store_n(p, (uns
 
 inline unsigned int* pack_counters(int s) { return G.counters + (size_t)s * kCounterWords; }
 inline unsigned int* done_counters(int s) { return G.counters + (size_t)(MAXSLOT + s) * kCounterWords; }
+inline unsigned int* wire_counters(int rail, int s) { return G.counters + ((size_t)2 * MAXSLOT + 1 + (size_t)rail * MAXSLOT + s) * kCounterWords; }
 inline unsigned long long* relay_word(int s) { return (unsigned long long*)(G.counters + (size_t)2 * MAXSLOT * kCounterWords) + (size_t)s * 8; }
 inline char* slot_send(int s) { return G.sendbase + (size_t)s * G.stride; }
 inline char* slot_recv(int s) { return G.recvbase + (size_t)s * G.stride; }
@@ -198,8 +201,10 @@ int configure(const char* devs, size_t cap);
 int init_impl(int rank, const char* devs, size_t cap);
 void teardown();
 void stop_progress();
-int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm = nullptr);
-int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm = nullptr);
+int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm = nullptr,
+                 PackArgs* hold = nullptr);
+int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, const Call& c, const NormArgs* nm = nullptr,
+                     const PackArgs* with_pack = nullptr);
 int flush_pending();
 void note_stream(void* stream, size_t nbytes);
 bool rails_idle();
@@ -209,6 +214,11 @@ int drain_rails();
 // The transfer of one rail's fragment of one call and the wait for the peer's fragment
 // (replaces do_xfer_rail, step4/libtbvcoll.cpp:172-211).  Returns 0, or -1 on error / watchdog.
 int wire_xfer(Rail& x, const Item& it);
+// Its two non-blocking halves (stream wire only, no test hooks), for a progress thread that keeps several
+// transfers in flight, and the bookkeeping of a completed one (t0 = post started, tp = post returned).
+int wire_post(Rail& x, const Item& it, bool* owns);
+bool wire_arrived(const Rail& x, const Item& it);
+void wire_done(Rail& x, const Item& it, double t0, double tp);
 // Whose payload plays the peer for call `c` of `nbytes`: sets *peer (null = mirror) and c->resident.
 int peer_assign(Call* c, size_t nbytes, int dtype, const char** peer);
 // Must this caller stream's calls be deposited by copy engines rather than a side stream?

@@ -38,6 +38,7 @@ struct SumArgs {
     // optional in-kernel gate: block-leaders poll *wait_flag until >= seq
     const unsigned long long* wait_flag;
     unsigned long long* relay;  // device word: block 0 polls wait_flag and republishes it here for the other blocks
+    bool b_uncached = false;    // `b` lies in uncached memory: passing the gate needs no cache invalidation
     unsigned long long seq;
     unsigned long long spin_limit_ticks;   // bound of the in-kernel wait, in ticks of the device's constant wall clock
     // optional completion word (latency probe / footprint): last block stores seq
@@ -71,6 +72,9 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, 
 // are done, the sum blocks read the local tensor themselves); same legality rule as launch_pack_sum, and
 // the bounce must be uncached (sigmode 0).
 hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+// One launch of the chunked pipeline: pack `p` (a later chunk; uncached bounce, completion word raised by its own
+// blocks) and sum `s` (an earlier chunk, optionally gated inside on s.wait_flag with s.relay) as two sets of blocks.
+hipError_t launch_pipe(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 // A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
 // blocks of 1024 lanes, one 16-byte vector per lane.
 static constexpr int kSmallCallMaxBlocks = 64;       // 1 MiB; 64 x 16 waves = an eighth of the GPU's wave slots

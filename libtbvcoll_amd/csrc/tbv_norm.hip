@@ -111,9 +111,9 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormA
     }
     if (MODE == 2) {
         grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
-        if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+        if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     } else if (MODE == 1 && g.wait_flag) {
-        gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp);
+        gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     }
     float ssq = 0.0f;
 #pragma unroll
@@ -198,6 +198,7 @@ hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const 
                      s.pre_word = p->pre.word; s.pre_seq = p->pre.seq; }
     else { s.pre_word = q.pre.word; s.pre_seq = q.pre.seq; s.fp = q.fp; }
     s.out = (u32x4*)q.out; s.b = (const u32x4*)q.b; s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks;
+    s.b_uncached = q.b_uncached;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.a = (const u32x4*)q.a; s.nbytes = q.nbytes; s.seq = q.seq;
     // Lanes per row: the fewest vectors per lane (1, 2, 4, 8) that bring a row down to 256 lanes, so that eight rows

@@ -155,6 +155,53 @@ int resident_refill(int form)
     return 0;
 }
 
+// Stream wire deposit of one rail fragment: side-stream copies of the fragment into the receive slot, then
+// the 64-bit arrival word on the same stream.  Nothing here waits.
+int stream_deposit(Rail& x, const Item& it, size_t off, size_t len, bool withheld)
+{
+    unsigned long long* aw = aflag(x.idx, it.slot);
+    const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
+    size_t n = len;
+    if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;   // staged payload has no tag
+    // One launch when the receive ring is uncached: the library's own copy kernel writes the fragment and its last
+    // block raises the arrival word, as the pack raises its completion word (stores to uncached memory are visible
+    // once acknowledged; into a cached ring the signal has to wait for the end of the copy kernel instead, below).
+    // Every HIP call of the three threads involved goes through the runtime's locks, so calls per transfer count.
+    if ((G.uncached & 2) && !G.chunkb && !(it.peer && G.tag)) {
+        PackArgs pa{};
+        pa.dst = slot_recv(it.slot) + off; pa.src = src; pa.nbytes = n; pa.seq = it.seq;
+        pa.cflag = withheld ? nullptr : aw; pa.arrive = wire_counters(x.idx, it.slot);
+        if (launch_pack(pa, x.wire) != hipSuccess) { LOGF("rail%d peer deposit failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
+        return 0;
+    }
+    // TBV_CHUNK: the fragment travels as several writes, the completion signal only after the last
+    // (step4/libtbvcoll.cpp:181-194)
+    const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
+    for (size_t o = 0; o < n; o += ck)
+        if (hipMemcpyAsync(slot_recv(it.slot) + off + o, src + o, std::min(ck, n - o), hipMemcpyDefault, x.wire) != hipSuccess) {
+            LOGF("rail%d peer deposit failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
+    if (it.peer && G.tag) {              // the peer's own tag travels at the end of its payload
+        size_t to = tag_offset(it.nbytes);
+        if (to >= off && to < off + len &&
+            stream_bump(x.wire, (unsigned long long*)(slot_recv(it.slot) + to), it.seq) != hipSuccess) return -1;
+    }
+    if (!withheld && stream_bump(x.wire, aw, it.seq) != hipSuccess) {
+        LOGF("rail%d arrival signal failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
+    return 0;
+}
+
+void account_arrival(Rail& x, const Item& it, double t0, double tp, double ta)
+{
+    record_arrival(it.seq, x.idx);
+    std::lock_guard<std::mutex> lk(G.smx);
+    x.rl_post += tp - t0; x.rl_arr += ta - t0; x.rl_n++;
+    if (x.idx == 0) {
+        G.t_acc += ta - t0; G.n_acc++;
+        int b = 0; { size_t v = it.nbytes; while (v >>= 1) b++; } if (b > 31) b = 31;
+        G.hb_t[b] += ta - t0; G.hb_n[b]++; G.hb_r[b] += (uint64_t)it.R;
+    }
+}
+
 void refresh_hooks()
 {
     int h = (!G.script.empty() || G.withhold_seq.load() != 0) ? 1 : 0;
@@ -217,22 +264,7 @@ int wire_xfer(Rail& x, const Item& it)
         if (host_deposit(x, it, off, len, t0) != 0) return -1;
         if (!withheld) st_rel(aw, it.seq);
     } else if (!it.resident) {
-        const char* src = it.peer ? it.peer + off : slot_send(it.slot) + off;
-        size_t n = len;
-        if (it.peer && off + n > it.nbytes) n = it.nbytes > off ? it.nbytes - off : 0;   // staged payload has no tag
-        // TBV_CHUNK: the fragment travels as several writes, the completion signal only after the last
-        // (step4/libtbvcoll.cpp:181-194)
-        const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
-        for (size_t o = 0; o < n; o += ck)
-            if (hipMemcpyAsync(slot_recv(it.slot) + off + o, src + o, std::min(ck, n - o), hipMemcpyDefault, x.wire) != hipSuccess) {
-                LOGF("rail%d peer deposit failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
-        if (it.peer && G.tag) {              // the peer's own tag travels at the end of its payload
-            size_t to = tag_offset(it.nbytes);
-            if (to >= off && to < off + len &&
-                stream_bump(x.wire, (unsigned long long*)(slot_recv(it.slot) + to), it.seq) != hipSuccess) return -1;
-        }
-        if (!withheld && stream_bump(x.wire, aw, it.seq) != hipSuccess) {
-            LOGF("rail%d arrival signal failed seq=%llu", x.idx, (unsigned long long)it.seq); return -1; }
+        if (stream_deposit(x, it, off, len, withheld) != 0) return -1;
     } else if (!withheld) {
         st_rel(aw, it.seq);                  // payload already in place: arrival is immediate
     }
@@ -246,20 +278,26 @@ int wire_xfer(Rail& x, const Item& it)
             return -1;
         }
     }
-    const double d = nowt() - t0;
-    record_arrival(it.seq, x.idx);
+    account_arrival(x, it, t0, tp, nowt());      // logged before the next rail in the script may go
     if (my_turn != (size_t)-1) G.turn.store(my_turn + 1, std::memory_order_release);
-    {
-        std::lock_guard<std::mutex> lk(G.smx);
-        x.rl_post += tp - t0; x.rl_arr += d; x.rl_n++;
-        if (x.idx == 0) {
-            G.t_acc += d; G.n_acc++;
-            int b = 0; { size_t v = it.nbytes; while (v >>= 1) b++; } if (b > 31) b = 31;
-            G.hb_t[b] += d; G.hb_n[b]++; G.hb_r[b] += (uint64_t)it.R;
-        }
-    }
     return 0;
 }
+
+// The two non-blocking halves of the stream wire, for a progress thread that keeps several transfers in
+// flight (a NIC with several work requests posted): post the deposit and its arrival signal; later ask
+// whether the signal has come.  *owns = false when this rail has no fragment of the call.
+int wire_post(Rail& x, const Item& it, bool* owns)
+{
+    size_t off = 0, len = 0;
+    *owns = rail_fragment(it.xbytes, it.R, x.idx, &off, &len);
+    if (!*owns) return 0;
+    if (it.resident) { st_rel(aflag(x.idx, it.slot), it.seq); return 0; }
+    return stream_deposit(x, it, off, len, false);
+}
+
+bool wire_arrived(const Rail& x, const Item& it) { return ld_acq(aflag(x.idx, it.slot)) >= it.seq; }
+
+void wire_done(Rail& x, const Item& it, double t0, double tp) { account_arrival(x, it, t0, tp, nowt()); }
 
 bool use_host_wire(hipStream_t st)
 {

@@ -164,7 +164,7 @@ MODES = {
     "sync": {"TBV_ASYNC": 0},
     "tag": {"TBV_TAG": 1},
     "cached_bounce": {"TBV_UNCACHED": 0},
-    "uncached_both": {"TBV_UNCACHED": 3},
+    "recv_cached": {"TBV_UNCACHED": 1},
     "railsum": {"TBV_RAILSUM": 1},
     "fusewait": {"TBV_FUSEWAIT": 1 << 30},
     "stream_gate_only": {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0, "TBV_ONEKERNEL": 0},
