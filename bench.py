@@ -21,6 +21,7 @@ from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also
                    workload, 10,000 back-to-back calls: library default (one kernel per
                    call) and, as decode_latency_stream_gate, the reference's sequence
                    pack kernel, hipStreamWaitValue64, sum kernel
+  host_cost_per_call   time inside tbv_ar_allreduce and of its last launch, idle and busy stream
   pipeline_64MiB_fp16  64 MiB fp16 as 16 chunks of 4 MiB over 2 rails x 4 slots
   cold_int8_codec      the cold step with the int8 payload codec on
   sum_rmsnorm_fusion   the sum fused with the following RMSNorm against the two kernels apart
@@ -104,8 +105,6 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
         t0 = time.perf_counter()
         for _ in range(k):
             step()
-        while not st.query():          # poll, so that the synchronize below returns at once instead of after a sleep
-            pass
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
@@ -224,6 +223,57 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
                         "host_enqueue_us is the time inside tbv_ar_allreduce per call, host_post_us its last launch"}
 
 
+def run_host_cost(tbv, torch, synth, st, calls=2000):
+    """Time inside tbv_ar_allreduce per call (enqueue) and of its last launch (post), from the library's own
+    statistics, when the caller is never held up by back-pressure: the stream is drained between calls (idle
+    stream) or the calls are issued back to back with the peer's payload already in place (busy stream, the
+    GPU work of these sizes is shorter than the host's)."""
+    import ctypes
+    out = {"what": "tbv_ar_stats' enqueue / post per call in us; idle = stream drained between calls, peer staged per call; "
+                   "busy = back to back, peer's payload resident, the caller never waits for ring room"}
+    for nb, name in ((N_DECODE, "8KB"), (4 << 20, "4MiB"), (N_PREFILL, "16MiB")):
+        for k in TUNING_KEYS:
+            os.environ.pop(k, None)
+        os.environ["TBV_NSLOT"] = "4"
+        tbv.shutdown()
+        tbv.init(0, "rail0", "", cap_bytes=nb)
+        a = torch.from_numpy(synth.normal(3, nb // 2)).to(torch.bfloat16).cuda()
+        b = torch.from_numpy(synth.normal(4, nb // 2)).to(torch.bfloat16).cuda()
+        o = torch.empty_like(a)
+        fn = tbv.raw_fn()
+        pa, po, ps = ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(o.data_ptr()), ctypes.c_void_p(st.cuda_stream)
+        res = {}
+        with torch.cuda.stream(st):
+            for _ in range(100):
+                tbv.stage_peer(b); fn(pa, po, nb, 2, ps); torch.cuda.synchronize()
+            tbv.stats4()
+            for _ in range(calls):
+                tbv.stage_peer(b); fn(pa, po, nb, 2, ps); torch.cuda.synchronize()
+            _, _, post, enq, _ = tbv.stats4()
+            res["idle"] = {"enqueue_us": round(enq, 2), "post_us": round(post, 2)}
+            if nb > (4 << 20):         # GPU-bound beyond this size: back-to-back calls wait for ring room
+                res["bit_exact"] = bool(torch.equal(o, a + b)) and not tbv.err()
+                out[name] = res
+                continue
+            tbv.peer_resident(b)
+            for _ in range(200):
+                fn(pa, po, nb, 2, ps)
+            torch.cuda.synchronize(); tbv.stats4()
+            t0 = time.perf_counter()
+            for _ in range(10 * calls):
+                fn(pa, po, nb, 2, ps)
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            _, _, post, enq, _ = tbv.stats4()
+            res["busy"] = {"enqueue_us": round(enq, 2), "post_us": round(post, 2), "caller_loop_us_per_call": round((t1 - t0) / (10 * calls) * 1e6, 2)}
+            res["bit_exact"] = bool(torch.equal(o, a + b)) and not tbv.err()
+            tbv.peer_resident(None)
+        out[name] = res
+    tbv.shutdown()
+    os.environ.pop("TBV_NSLOT", None)
+    return out
+
+
 def run_pipeline(tbv, torch, synth, st, reps=20):
     """64 MiB fp16 as 16 chunks of CAP = 4 MiB over 2 rails x 4 slots, each (chunk, rail) fragment deposited by a
     side-stream copy and signalled by a 64-bit flag; three packs ahead, so sums overlap arrivals."""
@@ -246,9 +296,11 @@ def run_pipeline(tbv, torch, synth, st, reps=20):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             tbv.all_reduce_chunked(a, out)
-            torch.cuda.synchronize()
+            st.synchronize()           # the caller's stream is complete: the result is there for whatever the caller queues next
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()   # (a device-wide wait also visits the rails' side streams: 50 us more, none of it the path's)
             if r >= 3:
-                times.append(time.perf_counter() - t0)
+                times.append(t1 - t0)
     ok = bool(torch.equal(out, a + p)) and not tbv.err()
     tbv.shutdown()
     os.environ.pop("TBV_NSLOT", None)
@@ -256,7 +308,7 @@ def run_pipeline(tbv, torch, synth, st, reps=20):
     return {"us": round(med * 1e6, 1), "min_us": round(min(times) * 1e6, 1), "GBps_5N": round(5 * numel * 2 / med / 1e9, 1),
             "bit_exact": ok, "reps": reps,
             "what": "tbv_ar_allreduce_chunked, 16 x 4 MiB fp16, 2 rails x NSLOT 4, every fragment through the emulated wire; "
-                    "host clock from the call to the stream's completion, median"}
+                    "host clock from the call to the completion of the caller's stream, median"}
 
 
 def run_rmsnorm_fusion(tbv, torch, synth, st):
@@ -330,7 +382,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
-    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,pipeline,codec,rmsnorm,cpu",
+    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,host,pipeline,codec,rmsnorm,cpu",
                     help="comma list of the extra legs to run beside the headline (cold) leg")
     ap.add_argument("--headline-env", default="", help="TBV_X=v,... applied to the headline leg (for profiling one variant)")
     ap.add_argument("--rotate", default=f"{COLD_NSLOT},{COLD_NBUF}",
@@ -437,6 +489,8 @@ def main():
     if "decode" in legs:
         line["decode_latency"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=True)
         line["decode_latency_stream_gate"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=False)
+    if "host" in legs:
+        line["host_cost_per_call"] = run_host_cost(tbv, torch, synth, st)
     if "pipeline" in legs:
         line["pipeline_64MiB_fp16"] = run_pipeline(tbv, torch, synth, st)
     if "codec" in legs:

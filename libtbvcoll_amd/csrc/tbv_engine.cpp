@@ -162,17 +162,19 @@ void* progress_rail(void* arg)
             continue;
         }
 
-        // post whatever is ready, in order
-        while (posted < head && !G.err.load(std::memory_order_relaxed)) {
+        // post the next one that is ready, in order; one per turn, so that an arrival is never left unseen behind
+        // several postings (a posting is a kernel launch, 3 us and more)
+        if (posted < head && !G.err.load(std::memory_order_relaxed)) {
             const Item& it = x.q[posted % NS];
-            if (it.host_wire || G.hooks) break;                      // that one goes one at a time, once it is the oldest
-            if (t_watch == 0) t_watch = nowt();
-            if (pack_complete(x, it, t_watch, NS) != 1) break;
-            const int k = (int)(posted % NS);
-            t_post0[k] = nowt();
-            if (wire_post(x, it, &owns[k]) != 0) { G.err.store(1); break; }
-            t_post1[k] = nowt();
-            posted++; t_watch = 0;
+            if (!it.host_wire && !G.hooks) {                         // else it goes one at a time, once it is the oldest
+                if (t_watch == 0) t_watch = nowt();
+                if (pack_complete(x, it, t_watch, NS) == 1) {
+                    const int k = (int)(posted % NS);
+                    t_post0[k] = nowt();
+                    if (wire_post(x, it, &owns[k]) != 0) G.err.store(1);
+                    else { t_post1[k] = nowt(); posted++; t_watch = 0; }
+                }
+            }
         }
         // finish the oldest one when its fragment has arrived
         if (posted > tail) {
@@ -550,7 +552,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         // place before the sum is even launched and the stream needs no gate at all.
         const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
         // (a row kernel has one block per row and no grid cap: it may only wait inside when its rows are few)
-        const bool fusewait = G.async && !arrived && (pipe || c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
+        const bool fusewait = G.async && !arrived && (pipe || c.held || c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
                               !(nm && nm->rows > (unsigned)kRowNormMaxSmallRows);
         if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
