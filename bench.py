@@ -364,16 +364,16 @@ def run_cpu_baseline(torch, synth):
     a = oracle.torch_bits(torch.from_numpy(synth.prefill_activations(100, n // 2)).to(torch.bfloat16)).copy()
     b = oracle.torch_bits(torch.from_numpy(synth.prefill_activations(101, n // 2)).to(torch.bfloat16)).copy()
     cores = max(1, min(16, os.cpu_count() or 1))
-    t1 = oracle.time_reduce_copy(oracle.DT_BF16, a, b, 1, 2, 40)
-    tn = oracle.time_reduce_copy(oracle.DT_BF16, a, b, cores, 5, 300)
+    t1 = oracle.time_reduce_copy(oracle.DT_BF16, a, b, 1, 2, 200)
+    tn = oracle.time_reduce_copy(oracle.DT_BF16, a, b, cores, 5, 2000)
     nd = N_DECODE
     da = oracle.torch_bits(torch.from_numpy(synth.normal(0, nd // 2)).to(torch.bfloat16)).copy()
     db = oracle.torch_bits(torch.from_numpy(synth.normal(1, nd // 2)).to(torch.bfloat16)).copy()
     td = oracle.time_reduce_copy(oracle.DT_BF16, da, db, 1, 100, 2000)
     return {"value": round(5 * n / tn / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
             "single_thread_GBps": round(5 * n / t1 / 1e9, 2), "decode_8KB_single_thread_us": round(td * 1e6, 2),
-            "sample": f"16 MiB bf16 prefill step (pack 2N + sum 3N), median of 300 steps on {cores} threads "
-                      f"(static contiguous partition) and of 40 steps on 1 thread; 8 KB decode step: median of 2000 on 1 thread"}
+            "sample": f"16 MiB bf16 prefill step (pack 2N + sum 3N), median of 2000 steps on {cores} threads "
+                      f"(static contiguous partition) and of 200 steps on 1 thread, about 10 s of CPU work; 8 KB decode step: median of 2000 on 1 thread"}
 
 
 def main():

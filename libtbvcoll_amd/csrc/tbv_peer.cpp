@@ -4,10 +4,12 @@
 // pairs set up by a TCP rendezvous (step4/libtbvcoll.cpp:172-224 transfer and reaping,
 // :343-403 bring-up).  Here the peer is played on the same GPU: for every call, each
 // rail's progress thread copies that rail's fragment of the peer payload into the receive
-// slot (side-stream hipMemcpyAsync, or a copy-engine transfer) and then raises a 64-bit
-// arrival word, the signal the immediate's completion gave.  wire_xfer() is the seam a
-// real transport would replace; everything else in this file feeds it (payload staging,
-// the early-peer mode, arrival scripts and withheld signals for tests).
+// slot (a copy kernel on the rail's side stream whose last block raises the arrival word;
+// side-stream copies plus a stream write into a cached ring; or a copy-engine transfer)
+// and the 64-bit arrival word is the signal the immediate's completion gave.  wire_xfer()
+// and its non-blocking halves wire_post() / wire_arrived() / wire_done() are the seam a
+// real transport would replace; everything else in this file feeds them (payload staging,
+// the early-peer mode, arrival scripts, held rails and withheld signals for tests).
 #include "tbv_engine.h"
 
 #include <sched.h>

@@ -163,6 +163,25 @@ def test_guards_and_return_codes(orc):
         assert tbv.seq() == 0                                        # nothing above consumed a sequence number
         # init is idempotent: a second call changes nothing
         assert tbv.lib().tbv_ar_init(1, b"a,b,c", b"", 1, 1 << 20) == 0 and tbv.lib().tbv_ar_cap() == 8192
+        # an empty call through the raw C function (the Python wrapper answers those itself): it takes a sequence
+        # number like any other call, touches nothing and leaves no error behind, in every launch form
+        keep = x.clone()
+        for k in range(1, 7):
+            assert fn(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(x.data_ptr()), 0, k % 3, ctypes.c_void_p(st)) == 0
+            assert tbv.seq() == k
+        torch.cuda.synchronize()
+        assert torch.equal(x, keep) and not tbv.err()
+    for env in ({"TBV_ONEKERNEL": 0}, {"TBV_FUSEWAIT": 0, "TBV_DEFERSIG": 0, "TBV_ONEKERNEL": 0}, {"TBV_ASYNC": 0}):
+        with session(rails=2, cap=8192, **env) as tbv:
+            fn = tbv.raw_fn()
+            x = torch.ones(16, device="cuda"); keep = x.clone()
+            for k in range(1, 6):
+                say("empty call", env, k)
+                assert fn(ctypes.c_void_p(x.data_ptr()), None, 0, 0, ctypes.c_void_p(st)) == 0
+            tbv.stage_peer(keep)
+            assert tbv.all_reduce(x)                                   # and the ring goes on working after them
+            torch.cuda.synchronize()
+            assert torch.equal(x, keep + keep) and not tbv.err() and tbv.seq() == 6
 
 
 def test_mirror_mode_and_send_slot_image(orc):
