@@ -315,6 +315,8 @@ int configure(const char* devs, size_t cap)
 {
     auto geti = [](const char* k, int d) { const char* e = getenv(k); return e ? atoi(e) : d; };
     auto getz = [](const char* k, size_t d) { const char* e = getenv(k); return e ? (size_t)strtoull(e, 0, 10) : d; };
+    // tbv_ar_cap() reports the cap as an int (step4/libtbvcoll.cpp:537): larger caps cannot be told to the caller
+    if (cap > (size_t)0x7ffff000) FAIL("cap %zu B is above what tbv_ar_cap can report (2 GiB - 4 KiB)", cap);
     G.cap = (cap + 4095) & ~(size_t)4095;
     G.async = geti("TBV_ASYNC", 1);
     G.gpusig = geti("TBV_GPUSIG", 1);

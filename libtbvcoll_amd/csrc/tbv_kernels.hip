@@ -96,12 +96,13 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 // local tensor into the bounce slot and count themselves complete (the pack's completion
 // word is raised as soon as those P blocks are done, not at the end of the kernel), the
 // remaining blocks sum.  Every kernel in a stream costs about 2.4 us of launch-to-launch
-// time on this GPU whatever it does, so the 16 MiB step drops from 15.2-16.0 us (two
-// launches) to 12.9-13.6 us on cache-cold buffers and from 10.9 to 9.6 us on resident
-// ones.  The sum blocks read the local tensor themselves (the step still moves 5 bytes
-// per payload byte, of which the second read of the local tensor usually hits the
-// Infinity Cache).  Only legal when the received payload is already in place: there is
-// no gate in this kernel.
+// time on this GPU whatever it does, so the 16 MiB step drops from 14.1 us (two launches)
+// to 12.7 us on cache-cold buffers and from 10.9 to 9.6 us on resident ones.  The sum
+// blocks read the local tensor themselves: the step still moves 5 bytes per payload byte,
+// but pack block b and sum block P+b work on the same vectors and, with P a multiple of
+// 8, land on the same XCD (blocks go to the eight XCDs round-robin), so the second read
+// is served by that XCD's L2 (counters: 4.007 bytes per payload byte cross the fabric).
+// Only legal when the received payload is already in place: there is no gate in this kernel.
 template <int DT, int UP, int US, bool STREAM>
 __global__ __launch_bounds__(kMaxSmallThreads) void k_merged(StepArgs g)
 {

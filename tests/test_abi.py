@@ -106,6 +106,18 @@ def test_configure_rejects_bad_rail_counts():
     lib.tbv_emu_shutdown()
 
 
+def test_configure_bounds_the_cap_by_what_tbv_ar_cap_can_report():
+    """tbv_ar_cap returns an int (step4/libtbvcoll.cpp:537): the largest cap is 2 GiB - 4 KiB, rounded like any other."""
+    lib = tbvcoll.load()
+    lib.tbv_emu_shutdown()
+    assert lib.tbv_emu_configure(b"a,b", (1 << 31) - 4096) == 0 and lib.tbv_ar_cap() == (1 << 31) - 4096
+    lib.tbv_emu_shutdown()
+    assert lib.tbv_emu_configure(b"a,b", (1 << 31) - 4095) == -1
+    lib.tbv_emu_shutdown()
+    assert lib.tbv_emu_configure(b"a,b", 1 << 40) == -1
+    lib.tbv_emu_shutdown()
+
+
 def test_binding_surface_matches_reference_module():
     for name in ("init", "all_reduce", "is_async", "err", "rails", "hist", "raw_fn", "cap", "stats", "stats3", "stats4",
                  "stats5"):

@@ -285,3 +285,46 @@ def test_nan_and_inf_propagation(orc, name):
         keep = ~nan.numpy()
         assert np.array_equal(g[keep], w[keep])
         assert int(torch.isinf(out).sum()) > 500
+
+
+def test_one_gibibyte_calls(orc):
+    """The largest sizes: 1 GiB calls (two rails of 512 MiB each, 64 Mi vectors per kernel) in two dtypes, in place and
+    out of place, and 1.5 GiB as two pipelined chunks.  Checked in full against the GPU's own add (bit-identical for
+    these types) and on both ends of the tensor against the CPU restatement."""
+    n = 1 << 30
+    with session(rails=2, cap=n, TBV_NSLOT=2) as tbv:
+        assert tbv.cap() == n
+        for name in ("bf16", "f32"):
+            dt = DT[name]
+            numel = n // torch.empty(0, dtype=dt).element_size()
+            g = torch.Generator(device="cuda"); g.manual_seed(77)
+            a = (torch.rand(numel, device="cuda", generator=g) * 8 - 4).to(dt)
+            b = (torch.rand(numel, device="cuda", generator=g) * 8 - 4).to(dt)
+            want = a + b
+            out = torch.empty_like(a)
+            say("1 GiB", name, "out of place")
+            tbv.stage_peer(b); assert tbv.all_reduce(a, out)
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int32), want.view(torch.int32)), name
+            k = 1 << 20
+            for sl in (slice(0, k), slice(numel - k, numel)):
+                assert first_diff(out[sl], oracle_sum(orc, a[sl], b[sl])) is None, name
+            say("1 GiB", name, "in place")
+            x = a.clone()
+            tbv.stage_peer(b); assert tbv.all_reduce(x)
+            torch.cuda.synchronize()
+            assert torch.equal(x.view(torch.int32), want.view(torch.int32)), name
+            del x, out, want
+        # 1.5 GiB over the 1 GiB cap: two chunks through the pipeline entry point
+        numel = 3 * (n // 4)
+        a = (torch.rand(numel, device="cuda") * 8 - 4).to(torch.bfloat16)
+        b = (torch.rand(numel, device="cuda") * 8 - 4).to(torch.bfloat16)
+        out = torch.empty_like(a)
+        per = n // 2
+        say("1.5 GiB chunked")
+        tbv.stage_peer(b[:per]); tbv.stage_peer(b[per:])
+        assert tbv.all_reduce(a, out) is False                   # over the cap: the plain call declines
+        assert tbv.all_reduce_chunked(a, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), (a + b).view(torch.int16))
+        assert not tbv.err()
