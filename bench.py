@@ -220,7 +220,8 @@ def run_decode(tbv, torch, synth, st, iters, fusewait):
             "gate": "one kernel per call: pack, completion word, flag poll, sum (library default up to 1 MiB)" if fusewait
             else "pack kernel, hipStreamWaitValue64, sum kernel (TBV_FUSEWAIT=0 TBV_DEFERSIG=0 TBV_ONEKERNEL=0)",
             "measured": "host clock: just before the progress thread raises the flag -> host sees the sum's done word; "
-                        "host_enqueue_us is the time inside tbv_ar_allreduce per call, host_post_us its last launch"}
+                        "host_enqueue_us is the time inside tbv_ar_allreduce per call in this back-to-back loop (it includes waiting for "
+                        "ring room behind the emulated wire), host_post_us its last launch; the *_idle_us pair is the same call on a drained stream"}
 
 
 def run_host_cost(tbv, torch, synth, st, calls=2000):
@@ -491,6 +492,10 @@ def main():
         line["decode_latency_stream_gate"] = run_decode(tbv, torch, synth, st, args.decode_iters, fusewait=False)
     if "host" in legs:
         line["host_cost_per_call"] = run_host_cost(tbv, torch, synth, st)
+        if "decode_latency" in line:      # the decode loop above runs back to back: its enqueue time includes waits for ring room
+            idle = line["host_cost_per_call"]["8KB"]["idle"]
+            line["decode_latency"]["host_enqueue_idle_us"] = idle["enqueue_us"]
+            line["decode_latency"]["host_post_idle_us"] = idle["post_us"]
     if "pipeline" in legs:
         line["pipeline_64MiB_fp16"] = run_pipeline(tbv, torch, synth, st)
     if "codec" in legs:

@@ -115,14 +115,24 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormA
     } else if (MODE == 1 && g.wait_flag) {
         gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     }
+    if (MODE >= 1) {
+        // all loads of the received row before the first store: `out` may alias anything, so a load placed after a
+        // store waits for it
+        u32x4 y[VPL];
+#pragma unroll
+        for (int v = 0; v < VPL; v++) {
+            const unsigned j = tid + (unsigned)v * lanes;
+            const u32x4 zero = {0, 0, 0, 0};
+            y[v] = j < hv ? g.b[row0 + j] : zero;
+        }
+#pragma unroll
+        for (int v = 0; v < VPL; v++) x[v] = add_vec<DT>(x[v], y[v]);   // lanes past the row: 0 + 0 = +0 in every type
+    }
     float ssq = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPL; v++) {
         const unsigned j = tid + (unsigned)v * lanes;
-        if (MODE >= 1 && j < hv) {
-            x[v] = add_vec<DT>(x[v], g.b[row0 + j]);
-            __builtin_nontemporal_store(x[v], g.out + row0 + j);
-        }
+        if (MODE >= 1 && j < hv) __builtin_nontemporal_store(x[v], g.out + row0 + j);
         float f[Row<DT>::EPV];
         Row<DT>::unpack(x[v], f);                            // lanes past the row hold zeros: they add nothing
 #pragma unroll
