@@ -65,10 +65,12 @@ inline bool queue_empty(const Rail& x)
 void release_gpu(const Item& it)
 {
     G.rails_done[it.slot].store(0u, std::memory_order_relaxed);
-    G.released[it.slot].store(it.seq, std::memory_order_release);
     const int probe = G.probe.load(std::memory_order_relaxed);
     const double t0 = probe ? nowt() : 0.0;
     st_rel(gflag(it.slot), it.seq);
+    // only now may the caller reuse the slot: an early peer's call raises this same flag to its own, higher
+    // sequence number on entry, and that store must not be overtaken by the one above
+    G.released[it.slot].store(it.seq, std::memory_order_release);
     if (probe && !G.err.load()) {
         const unsigned long long* dw = doneword(it.slot);
         double t1 = t0;
