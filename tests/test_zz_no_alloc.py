@@ -97,3 +97,50 @@ def test_no_alloc_step_without_init():
         torch.cuda.synchronize()
         assert torch.equal(out, a + b) and torch.equal(bounce.view(torch.int16), a.view(torch.int16))
         assert int(words[0]) == seq and int(words[8]) == seq
+
+
+@pytest.mark.parametrize("uncached", [0, 1])
+def test_no_alloc_step_in_a_graph(uncached):
+    """Recorded into a HIP graph (the callers the entry point is for) and replayed four times with the program's own
+    eager work and synchronisations in between; every replay checked against the eager result.  With an uncached
+    bounce (a send slot of the initialised library) the step is the one-launch form, else pack kernel + sum kernel."""
+    from libtbvcoll_amd import tbvcoll
+    tbvcoll.shutdown()
+    lib = tbvcoll.load()
+    if uncached:
+        tbvcoll.init(0, "rail0", "", cap_bytes=4 << 20)
+    n = (2 << 20) + 64
+    a = dev(synth.uniform(15, n // 2), torch.bfloat16); b = dev(synth.uniform(16, n // 2), torch.bfloat16)
+    out = torch.empty_like(a); bounce = torch.empty_like(a)
+    bptr = lib.tbv_emu_send_slot(1) if uncached else bounce.data_ptr()
+    hip = _hip()
+    words = torch.zeros(16, dtype=torch.int64).pin_memory()
+    eager = torch.cuda.current_stream().cuda_stream
+    # first call outside any capture: it looks up the counters' address on this device
+    assert lib.tbv_step_noalloc(out.data_ptr(), a.data_ptr(), b.data_ptr(), bptr, uncached, n, 2,
+                                words.data_ptr(), words.data_ptr() + 64, 1, eager) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + b)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    say("capture")
+    with torch.cuda.graph(graph, stream=side):
+        rc = lib.tbv_step_noalloc(out.data_ptr(), a.data_ptr(), b.data_ptr(), bptr, uncached, n, 2,
+                                  words.data_ptr(), words.data_ptr() + 64, 7, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    for k in range(4):
+        # the program's own eager work and a synchronisation between replays; new inputs each time
+        a.copy_(dev(synth.uniform(20 + k, n // 2), torch.bfloat16)); b.mul_(0.5)
+        out.zero_(); bounce.zero_(); words.zero_()
+        if uncached:
+            assert hip.hipMemcpy(bptr, bounce.data_ptr(), n, 3) == 0
+        torch.cuda.synchronize()
+        say("replay", k)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, a + b), k
+        if uncached:
+            assert hip.hipMemcpy(bounce.data_ptr(), bptr, n, 3) == 0
+        assert torch.equal(bounce.view(torch.int16), a.view(torch.int16)), k
+        assert int(words[0]) == 7 and int(words[8]) == 7, k
+    tbvcoll.shutdown()
