@@ -48,7 +48,8 @@ int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_
  * in place.  Asynchronous: the result is valid in `stream` order.  Returns 0;
  * -2 when nbytes exceeds the cap (caller falls back to its own collective);
  * -1 when not initialised, after any earlier transfer error (sticky), or on a
- * launch failure.  One caller thread at a time.
+ * launch failure.  One caller thread at a time: a call that arrives while another
+ * thread is inside the library is refused with -1.
  */
 int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype, void* stream);
 

@@ -12,6 +12,18 @@ using namespace tbv;
 
 // ========================================================================== part 1: the drop-in boundary
 
+namespace {
+// The sequence number, the ring slots and the rails' queues have one producer (as in the reference, which
+// increments its sequence number without a lock, step4/libtbvcoll.cpp:435): calls may come from any thread, but
+// from one at a time.  Two at once would share a slot; say so instead.
+struct OneCaller {
+    bool ok;
+    OneCaller() : ok(G.in_call.exchange(1, std::memory_order_acquire) == 0) {}
+    ~OneCaller() { if (ok) G.in_call.store(0, std::memory_order_release); }
+};
+}  // namespace
+#define ONE_CALLER() OneCaller one_caller; if (!one_caller.ok) FAIL("two threads inside the library at once: calls must come from one thread at a time")
+
 extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_t cap)
 {
     (void)peer_ip; (void)port;
@@ -28,6 +40,7 @@ extern "C" int tbv_ar_allreduce(void* ptr, void* outp, size_t nbytes, int dtype,
     if (nbytes > G.cap) return -2;                    // caller falls back to its own collective
     if (dtype < 0 || dtype > 2) FAIL("unknown dtype %d", dtype);
     if (G.async && !G.run.load(std::memory_order_relaxed)) FAIL("progress threads were stopped by tbv_ar_fini");
+    ONE_CALLER();
     if (!outp) outp = ptr;
     hipStream_t st = (hipStream_t)stream;
     note_stream(stream, nbytes);
@@ -218,6 +231,7 @@ extern "C" int tbv_ar_allreduce_chunked(void* ptr, void* outp, size_t nbytes, in
     if (!G.run.load()) FAIL("progress threads were stopped by tbv_ar_fini");
     if (!outp) outp = ptr;
     if (nbytes == 0) return 0;
+    ONE_CALLER();
     hipStream_t st = (hipStream_t)stream;
     note_stream(stream, nbytes);
     const size_t esz = dtype == 0 ? 4 : 2;
@@ -268,6 +282,7 @@ extern "C" int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, con
     if (!outp) outp = ptr;
     if (((uintptr_t)ptr | (uintptr_t)outp | (uintptr_t)normed | (uintptr_t)weight) & 15) FAIL("rmsnorm buffers must be 16-byte aligned");
     if (G.async && !G.run.load(std::memory_order_relaxed)) FAIL("progress threads were stopped by tbv_ar_fini");
+    ONE_CALLER();
     hipStream_t st = (hipStream_t)stream;
     note_stream(stream, nbytes);
     NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};

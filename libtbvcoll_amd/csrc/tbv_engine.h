@@ -104,6 +104,7 @@ struct Engine {
     pthread_cond_t cv_item = PTHREAD_COND_INITIALIZER;    // caller -> progress: new item
     pthread_cond_t cv_room = PTHREAD_COND_INITIALIZER;    // progress -> caller: room in the ring
     std::atomic<int> caller_napping{0};                   // the caller is (about to be) asleep on cv_room
+    std::atomic<int> in_call{0};                          // a thread is inside one of the all-reduce entry points
     void* last_stream = nullptr;
     hipEvent_t switch_ev = nullptr;           // orders a new caller stream behind the previous one
     uint64_t n_stream_sw = 0;

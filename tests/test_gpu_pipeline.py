@@ -1,6 +1,8 @@
 """GPU tests of the protocol around the kernels: multi-rail chunked pipeline with a
 seeded arrival order, the async stress mix, the watchdog, and every mode switch."""
+import ctypes
 import os
+import threading
 import time
 
 import numpy as np
@@ -344,10 +346,20 @@ def test_early_peer_cannot_release_a_call_still_waiting_for_rail_1(orc):
         for k in range(nslot - 1):
             assert tbv.all_reduce(smalls[k], outs[k])          # seq 2..NSLOT: early peer, one rail, other slots
         lifter = threading.Timer(0.06, lambda: tbv.hold_rail(1, False))
+        # while this thread waits inside the library, a call from another thread is refused (one caller at a time)
+        # instead of sharing the sequence counter and the ring with it
+        intruder_rc = []
+        fn = tbv.raw_fn()
+        spare = torch.zeros(64, device="cuda")
+        stream_handle = torch.cuda.current_stream().cuda_stream
+        intruder = threading.Timer(0.02, lambda: intruder_rc.append(
+            fn(ctypes.c_void_p(spare.data_ptr()), None, 256, 0, ctypes.c_void_p(stream_handle))))
         t0 = time.time()
-        lifter.start()
+        lifter.start(); intruder.start()
         assert tbv.all_reduce(smalls[nslot - 1], outs[nslot - 1])   # seq 1+NSLOT wraps onto slot 1: waits for call 1's release
         waited = time.time() - t0
+        intruder.join()
+        assert intruder_rc == [-1], intruder_rc
         for k in range(nslot, len(smalls)):
             assert tbv.all_reduce(smalls[k], outs[k])
         lifter.join()
