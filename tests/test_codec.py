@@ -27,6 +27,19 @@ def parse_image(img, n):
     return hdr[:, :, 0].reshape(-1)[:G], hdr[:, :, 1].reshape(-1)[:G], codes
 
 
+def test_library_and_restatement_agree_on_image_sizes():
+    """The size of an image is host arithmetic in the library (no GPU needed): 2176 bytes per started superblock of
+    2048 elements, the same as the CPU restatement says and as the format's closed form."""
+    from libtbvcoll_amd import tbvcoll
+    lib = tbvcoll.load()
+    for code, esz in ((0, 4), (1, 2), (2, 2)):
+        for n in (0, 1, 127, 128, 2047, 2048, 2049, 100000, 8 << 20):
+            want = (n + 2047) // 2048 * 2176
+            assert lib.tbv_emu_codec_image_bytes(n * esz, code) == want
+            assert int(oracle.lib().orc_q8_image_bytes(n)) == want
+    assert lib.tbv_emu_codec_image_bytes(4096, 5) == 0              # unknown dtype
+
+
 @pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("n", [128, 2048, 2048 * 3 + 128 * 5 + 8, 100000])
 def test_codec_invariants(name, n):
