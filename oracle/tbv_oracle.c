@@ -17,6 +17,11 @@
  * force, exhaustive sweeps against numpy float16, a host compile of the HIP
  * headers' own operator+, and committed golden vectors.
  * Parity unpinned: NaN payload and sign of a NaN result (configs are finite).
+ *
+ * Further down: the ring/release model (pinned by an independent simulator's traces
+ * and a hand-worked scenario), the sum fused with RMSNorm and the int8 payload codec
+ * (neither exists in the reference; each carries its own note on what pins it).
+ * Parity unpinned there: the codec on non-finite inputs.
  */
 #include <stdint.h>
 #include <stddef.h>
