@@ -87,6 +87,37 @@ class Intercept:
             self.counters["fallback"] += 1
         return self.orig(group, input_)
 
+    def all_reduce_rmsnorm(self, group, input_, weight, eps):
+        """The tensor-parallel all-reduce of `input_` and the RMSNorm of its result (what every decoder layer does
+        next; the reference plans the fusion, reports/12_references.md:136): returns (reduced, normed).  Goes through
+        `tbv_ar_allreduce_rmsnorm` when the library takes the call (TP group, supported dtype and layout, rows of at
+        most 64 KiB, payload within the cap); otherwise the all-reduce goes the usual way (library or original) and the
+        norm is computed here in fp32, the formula vLLM's own kernel implements.  The fused kernel's `normed` is
+        within 2 ulp of that formula, so an output-hash comparison between a fused and an unfused run may differ."""
+        if group.world_size > 1 and self.tp_name is None:
+            try:
+                self.tp_name = self.ps.get_tp_group().unique_name
+            except Exception:
+                self.tp_name = False
+        fused = getattr(self.lib, "all_reduce_rmsnorm", None)
+        if (fused is not None and group.world_size > 1 and self.tp_name and group.unique_name == self.tp_name
+                and input_.dtype in _DT and input_.is_contiguous() and input_.dim() >= 1
+                and weight.dtype is input_.dtype and weight.is_contiguous() and weight.numel() == input_.shape[-1]):
+            if self.fn is None:
+                self._init()
+            t0 = time.perf_counter()
+            out = torch.empty_like(input_)
+            normed = fused(input_, weight, eps, out=out)
+            self.counters["py"] += time.perf_counter() - t0
+            if normed is not None:
+                self.counters["n"] += 1
+                self.counters["fused_norm"] = self.counters.get("fused_norm", 0) + 1
+                return out, normed
+        reduced = self._all_reduce(group, input_)
+        x = reduced.float()
+        normed = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)).to(reduced.dtype) * weight
+        return reduced, normed
+
     def report(self):
         """Counters plus the library's per-call averages (resets the latter), as the reference prints at the end."""
         r = dict(self.counters)

@@ -93,6 +93,46 @@ def test_routing_fallback_and_accounting(no_cuda_stream):
     assert ps.GroupCoordinator.all_reduce is ic.orig
 
 
+def test_fused_norm_routing_and_fallback(no_cuda_stream):
+    """all_reduce_rmsnorm: the fused entry point for the TP group when the library takes the call, else the plain
+    all-reduce (library or original) followed by the fp32 formula; both give (reduced, normed)."""
+    ps = make_ps(lambda t: torch.ones_like(t))
+    lib = FakeLib(cap=1 << 20)
+    taken = []
+
+    def fused(t, weight, eps, out=None):
+        taken.append((tuple(t.shape), eps))
+        if t.shape[-1] > 64:                      # plays "rows too long": the library declines
+            return None
+        out.copy_(t + 1)
+        return torch.full_like(t, 5.0)
+
+    lib.all_reduce_rmsnorm = fused
+    ic = vllm_intercept.install(ps, rank=0, devs="a", cap_bytes=1 << 20, lib=lib)
+    try:
+        w = torch.full((8,), 2.0)
+        x = torch.arange(16.0).reshape(2, 8)
+        red, nrm = ic.all_reduce_rmsnorm(ps.tp, x, w, 1e-6)
+        assert taken == [((2, 8), 1e-6)] and torch.equal(red, x + 1) and torch.equal(nrm, torch.full_like(x, 5.0))
+        assert ic.counters["fused_norm"] == 1 and ic.counters["n"] == 1 and ps.tp.orig_calls == 0
+        # declined by the library: plain all-reduce through the library's raw function, norm by the formula
+        big = torch.ones(2, 128)
+        red, nrm = ic.all_reduce_rmsnorm(ps.tp, big, torch.full((128,), 2.0), 0.0)
+        assert len(taken) == 2 and lib.calls[-1] == (2 * 128 * 4, 0) and ic.counters["fused_norm"] == 1
+        # another group: the original all-reduce, then the formula (x + 1 = 2 everywhere: rms 2, normed 1 * weight)
+        red, nrm = ic.all_reduce_rmsnorm(ps.pp, torch.ones(2, 8), w, 0.0)
+        assert ps.pp.orig_calls == 1 and torch.equal(red, torch.full((2, 8), 2.0)) and torch.allclose(nrm, torch.full((2, 8), 2.0))
+        # world size 1: nothing to reduce, the norm is still computed
+        red, nrm = ic.all_reduce_rmsnorm(ps.single, torch.full((1, 8), 3.0), w, 0.0)
+        assert torch.equal(red, torch.full((1, 8), 3.0)) and torch.allclose(nrm, torch.full((1, 8), 2.0))
+        # a weight of another dtype or length is not handed to the library
+        n_before = len(taken)
+        ic.all_reduce_rmsnorm(ps.tp, x, torch.full((8,), 2.0, dtype=torch.float64), 1e-6)
+        assert len(taken) == n_before
+    finally:
+        ic.uninstall()
+
+
 def test_rank0_passes_no_peer_address_and_eager_init(no_cuda_stream):
     ps = make_ps(lambda t: t)
     lib = FakeLib()
@@ -160,3 +200,42 @@ def test_toy_decode_loop_hash_matches_fallback():
         assert got == want, (ids[0][:8], ids_ref[0][:8])
         assert not tbvcoll.err()
 
+
+
+@pytest.mark.gpu
+def test_fused_norm_through_the_real_library():
+    """all_reduce_rmsnorm of the intercept on the GPU: the reduced tensor and the normalised one equal the CPU
+    restatement bit for bit when the library takes the call; rows it does not take come back from the fallback
+    formula within 2 ulp of that restatement."""
+    import numpy as np
+    from gpu_util import bits_np, session
+    from libtbvcoll_amd import synth, tbvcoll
+    from oracle import oracle
+    hidden, rows = 4096, 16
+    a = torch.from_numpy(synth.normal(31, rows * hidden)).to(torch.bfloat16).reshape(rows, hidden)
+    b = torch.from_numpy(synth.normal(32, rows * hidden)).to(torch.bfloat16).reshape(rows, hidden)
+    w = torch.from_numpy(1.0 + 0.25 * synth.normal(33, hidden)).to(torch.bfloat16)
+    want_out, want_normed = oracle.sum_rmsnorm(oracle.DT_BF16, bits_np(a), bits_np(b), bits_np(w), hidden, 1e-6)
+    with session(rails=2, cap=1 << 20):
+        tbvcoll.shutdown()
+        peer = {}
+        ps = make_ps(lambda t: peer["t"])
+        ic = vllm_intercept.install(ps, rank=0, devs="rail0,rail1", cap_bytes=1 << 20, eager=True)
+        try:
+            A, B, W = a.cuda(), b.cuda(), w.cuda()
+            tbvcoll.stage_peer(B)
+            red, nrm = ic.all_reduce_rmsnorm(ps.tp, A, W, 1e-6)
+            torch.cuda.synchronize()
+            assert np.array_equal(bits_np(red).reshape(-1), want_out) and np.array_equal(bits_np(nrm).reshape(-1), want_normed)
+            assert ic.counters["fused_norm"] == 1 and ps.tp.orig_calls == 0
+            # a strided view is taken neither by the fused entry point nor by the plain one: original all-reduce + formula
+            peer["t"] = B[:, ::2]
+            red2, nrm2 = ic.all_reduce_rmsnorm(ps.tp, A[:, ::2], W[::2].contiguous(), 1e-6)
+            torch.cuda.synchronize()
+            x = (A[:, ::2] + B[:, ::2]).float()
+            ref = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16) * W[::2]
+            assert ps.tp.orig_calls == 1 and ic.counters["fallback"] == 1
+            assert torch.equal(red2, A[:, ::2] + B[:, ::2]) and torch.equal(nrm2, ref)
+        finally:
+            ic.uninstall()
+        assert not tbvcoll.err()
