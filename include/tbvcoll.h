@@ -243,7 +243,7 @@ int tbv_step_noalloc(void* out, const void* local, const void* received, void* b
 
 /* What plain streaming kernels reach on this GPU, as measured denominators beside the
  * published HBM peak (no counterpart in the reference).  tbv_emu_hbm_probe streams
- * `bytes` per launch (kind 0 read, 1 write, 2 copy with non-temporal accesses, 3 plain
+ * `bytes` per launch (kind 0 read, 1 write, 2 copy with non-temporal loads, 3 plain
  * copy) `reps` times through successive windows of a pool of `pool_bytes` that it
  * allocates and frees itself, and returns the mean and minimum launch duration in
  * microseconds.  tbv_emu_launch_floor returns the launch-to-launch time of an empty

@@ -146,8 +146,10 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
         if (mode == 1) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
         bool last = true;
         if (nblk > 1) {
-            const unsigned g = bid / kGroup, ngroups = (nblk + kGroup - 1) / kGroup;
-            const unsigned pop = min(kGroup, nblk - g * kGroup);
+            // groups of 32 blocks; of 64 when the grid is larger than 32 groups' lines can count
+            const unsigned G = nblk > kGroup * (kCounterWords / kCtrLine - 1) ? 2 * kGroup : kGroup;
+            const unsigned g = bid / G, ngroups = (nblk + G - 1) / G;
+            const unsigned pop = min(G, nblk - g * G);
             unsigned int* gc = ctr + kCtrLine * (1 + g);
             last = false;
             if (__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == pop - 1) {

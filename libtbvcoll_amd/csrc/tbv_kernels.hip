@@ -295,7 +295,7 @@ void set_tuning(int unroll, int grid_cap, int block, int streaming)
     g_block = (block == 512 || block == 1024) ? block : kThreads;
     g_unroll = (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) ? unroll : 0;
     // the completion counters have one line per group of kGroup blocks: keep the grid within them
-    const int most = (int)(kGroup * (kCounterWords / kCtrLine - 1));
+    const int most = (int)(2 * kGroup * (kCounterWords / kCtrLine - 1));
     g_grid_cap = grid_cap >= 1 ? (grid_cap < most ? grid_cap : most) : 1024;
     g_grid_cap_given = grid_cap >= 1;
     g_stream = streaming != 0;
