@@ -488,3 +488,31 @@ def test_seeded_mix_of_everything(orc, seed, env):
                         assert first_diff(o, oracle_sum(orc, ka, ka if pp is None else pp)) is None
                 pend = []
         assert not tbv.err()
+
+
+def test_grids_beyond_the_small_counter_groups(orc):
+    """Grids of more than 4064 blocks count their completion in groups of 64 instead of 32 (the tuning knobs allow up
+    to 8128 blocks): pack, merged launch and sum at that size, staged and early peer, completion words included."""
+    n = 32 << 20
+    with session(rails=2, cap=n, TBV_UNROLL=1, TBV_GRIDCAP=8128, TBV_NSLOT=2) as tbv:
+        a = dev(synth.uniform(61, n // 2, -4.0, 4.0), torch.bfloat16)
+        b = dev(synth.uniform(62, n // 2, -4.0, 4.0), torch.bfloat16)
+        want = a + b
+        for k in range(3):
+            out = torch.empty_like(a)
+            say("8128-block grids, staged", k)
+            tbv.stage_peer(b)
+            assert tbv.all_reduce(a, out)
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+        tbv.peer_resident(b)
+        for k in range(3):
+            out = torch.empty_like(a)
+            say("8128-block grids, early peer", k)
+            assert tbv.all_reduce(a, out)
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+        tbv.peer_resident(None)
+        sl = slice(0, 1 << 20)
+        assert first_diff(out[sl], orc.sum_torch(a[sl].cpu(), b[sl].cpu())) is None
+        assert not tbv.err()
