@@ -43,7 +43,7 @@ N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
 COLD_NSLOT, COLD_NBUF = 16, 12         # 2 x 16 x 16 MiB of rings + 2 x 12 x 16 MiB of tensors = 896 MiB
 TRAFFIC_FILE = os.path.join("profiles", "prefill16MiB_cold_pmc_fetch_write.txt")
-TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL", "TBV_CODEC", "TBV_CODEC_MIN")
+TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_MERGEMAX", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL", "TBV_CODEC", "TBV_CODEC_MIN")
 
 
 def pct(xs, q):

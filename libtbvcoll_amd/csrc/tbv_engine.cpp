@@ -348,6 +348,7 @@ int configure(const char* devs, size_t cap)
     G.R = count_rails(devs);
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
     G.merge = geti("TBV_MERGE", 1);
+    G.merge_max = getz("TBV_MERGEMAX", (size_t)256 << 20);
     G.codec = geti("TBV_CODEC", 0);
     G.codec_min = getz("TBV_CODEC_MIN", (size_t)512 << 10);
     // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
@@ -405,7 +406,10 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                                     (nm ? nm->rows <= (unsigned)kRowNormMaxSmallRows : small_call_blocks(nbytes) <= kSmallCallMaxBlocks);
             // Payload already in place and too large for the one-kernel call: pack blocks and sum blocks in one
             // launch (a launch costs about 2.4 us of stream time whatever it does).
-            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && plain && G.packsig == 0 && !nm;
+            // (up to a size: the two halves share the local tensor through the L2 only while they stay close in time;
+            // at 1 GiB the merged launch moves 5.1-5.45 TB/s, two launches 5.6)
+            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && plain && G.packsig == 0 && !nm &&
+                                   nbytes <= G.merge_max;
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its

@@ -249,6 +249,8 @@ __global__ void k_fill_u32(unsigned int* p, unsigned int v, size_t n)
 // 4096) or 512/1024-lane blocks change nothing; fewer (256, 512) lose 10-40 %.
 
 static int g_unroll = 0;        // vectors per lane per iteration for the large path; 0 = the profile's choice
+// the completion counters have one line per group of blocks (32, or 64 for the largest grids): no grid may be larger
+static constexpr int kMostBlocks = (int)(2 * kGroup * (kCounterWords / kCtrLine - 1));
 static int g_grid_cap = 1024;
 static bool g_grid_cap_given = false;   // a cap from the environment applies to every launch shape
 static int g_block = kThreads;
@@ -273,11 +275,16 @@ static Geom geom_for(size_t nbytes, bool writeback = false, bool merged = false)
     else if (merged) {
         // the halves of a merged launch run side by side and do best when every block makes a single pass of two
         // vectors per lane (16 MiB, cold / resident: 12.75 / 9.55 us against 13.05 / 10.2 with 1024 blocks of one)
+        // (32 - 256 MiB: one pass of up to 8128 blocks per half 7.1-7.2 TB/s on 5N, 2048 looping blocks 6.8-7.05)
         g.unroll = nvec >= (size_t)2 * g_block * 1024 ? 2 : 1;
-        if (!g_grid_cap_given) cap = 2048;
+        if (!g_grid_cap_given) cap = kMostBlocks;
+    } else {
+        // the streaming profile keeps four loads per lane in flight, as long as that still leaves a block for every
+        // grid position, and makes one pass where the counters can count the blocks (64 MiB two-launch step 50.6 ->
+        // 49.2 us, 256 MiB 194.9 -> 189.5 us); the resident profile keeps to four blocks per CU
+        g.unroll = (g_stream && nvec >= (size_t)4 * g_block * g_grid_cap) ? 4 : 1;
+        if (g_stream && !g_grid_cap_given) cap = kMostBlocks;
     }
-    // the streaming profile keeps four loads per lane in flight, as long as that still leaves a block for every grid position
-    else g.unroll = (g_stream && nvec >= (size_t)4 * g_block * g_grid_cap) ? 4 : 1;
     // an L2 write-back per block is dear and they run one after another: use one fat block per CU
     if (writeback) { cap = 256; g.unroll = 8; }
     size_t tile = (size_t)g.block * g.unroll;
@@ -294,9 +301,7 @@ void set_tuning(int unroll, int grid_cap, int block, int streaming)
 {
     g_block = (block == 512 || block == 1024) ? block : kThreads;
     g_unroll = (unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) ? unroll : 0;
-    // the completion counters have one line per group of kGroup blocks: keep the grid within them
-    const int most = (int)(2 * kGroup * (kCounterWords / kCtrLine - 1));
-    g_grid_cap = grid_cap >= 1 ? (grid_cap < most ? grid_cap : most) : 1024;
+    g_grid_cap = grid_cap >= 1 ? (grid_cap < kMostBlocks ? grid_cap : kMostBlocks) : 1024;
     g_grid_cap_given = grid_cap >= 1;
     g_stream = streaming != 0;
 }

@@ -10,7 +10,7 @@ from libtbvcoll_amd import synth, tbvcoll
 
 TBV_KEYS = ("TBV_ASYNC", "TBV_GPUSIG", "TBV_KWAIT", "TBV_NSLOT", "TBV_CHUNK", "TBV_RAIL1MAX", "TBV_CPU", "TBV_WDOG",
             "TBV_TAG", "TBV_UNCACHED", "TBV_RAILSUM", "TBV_FUSE", "TBV_FUSEWAIT", "TBV_UNROLL", "TBV_GRIDCAP", "TBV_BLOCK",
-            "TBV_PACKSIG", "TBV_DEFERSIG", "TBV_WIRE", "TBV_ONEKERNEL", "TBV_MERGE", "TBV_STREAMING", "TBV_CODEC", "TBV_CODEC_MIN")
+            "TBV_PACKSIG", "TBV_DEFERSIG", "TBV_WIRE", "TBV_ONEKERNEL", "TBV_MERGE", "TBV_MERGEMAX", "TBV_STREAMING", "TBV_CODEC", "TBV_CODEC_MIN")
 DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 
 
