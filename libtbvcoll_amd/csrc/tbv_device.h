@@ -161,7 +161,13 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
                 }
             }
         }
-        if (last) store_sys(word, seq);
+        // Modes 1 and 2 have written the L2 back above.  In mode 0 the counted stores went to uncached memory and
+        // every wave waited for their acknowledgements before its block was counted, so they are in memory already:
+        // a release here would only make this wave write back an L2 that holds none of them.
+        if (last) {
+            if (mode == 0) __hip_atomic_store(word, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            else store_sys(word, seq);
+        }
     }
 }
 
