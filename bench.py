@@ -10,9 +10,14 @@ The headline (`value`, `roofline`) is the HBM-bound form of that step: 16 ring s
 and 12 rotating local/output tensors, 896 MiB touched in turn, so every operand comes
 from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also carries
 
+  region           what the timed region costs beside its steps (start and stop latency of a drained
+                   stream), from a second region of twice the steps
   long_run         the same leg over 2000 steps when --steps is small
   cold_two_launches, cold_fused_4N   the same cold step as pack kernel + sum kernel, and
                    as one kernel that reads the local tensor once (4N)
+  cold_staged      the same cold step when the peer's payload is NOT there yet: deposited per call
+                   through the emulated wire (one launch: pack blocks + gated sum blocks), and
+                   cold_gated_flag_up, that launch with its flag already up
   resident         the step with everything it touches resident in the Infinity Cache
                    (4 slots, one local/output tensor): a cache figure, labelled so
   achievable       what plain read / write / copy kernels reach on this GPU (1 GiB
@@ -43,7 +48,9 @@ N_PREFILL = 16 << 20                   # 2048 x 4096 bf16
 N_DECODE = 8192                        # 1 x 4096 bf16
 COLD_NSLOT, COLD_NBUF = 16, 12         # 2 x 16 x 16 MiB of rings + 2 x 12 x 16 MiB of tensors = 896 MiB
 TRAFFIC_FILE = os.path.join("profiles", "prefill16MiB_cold_pmc_fetch_write.txt")
-TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_MERGEMAX", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL", "TBV_CODEC", "TBV_CODEC_MIN")
+TRACE_FILE = os.path.join("profiles", "prefill16MiB_cold_kernel_trace.txt")
+TUNING_KEYS = ("TBV_NSLOT", "TBV_FUSE", "TBV_MERGE", "TBV_MERGEMAX", "TBV_STREAMING", "TBV_FUSEWAIT", "TBV_DEFERSIG", "TBV_ONEKERNEL", "TBV_CODEC", "TBV_CODEC_MIN",
+               "TBV_STAGEDMERGE", "TBV_FORCEGATE", "TBV_GATEDGRID", "TBV_GATEDUNROLL", "TBV_ROWGRID", "TBV_CODECGRID")
 
 
 def pct(xs, q):
@@ -65,16 +72,31 @@ def traffic_from_profile(kernel):
     return None
 
 
+def avg_from_profile(kernel):
+    """Average duration (us) of `kernel` as the committed rocprofv3 kernel-trace summary states it
+    (a line `KERNEL_AVG kernel=<name> avg_ns=<n> ...`); None when the file has no such line."""
+    try:
+        with open(os.path.join(ROOT, TRACE_FILE)) as f:
+            for ln in f:
+                m = re.match(r"\s*KERNEL_AVG kernel=(\S+) avg_ns=([0-9.]+)", ln)
+                if m and m.group(1) == kernel:
+                    return float(m.group(2)) / 1e3
+    except OSError:
+        pass
+    return None
+
+
 def own_warmup(warmup, nslot, nbuf):
     """Untimed steps before the clock: at least two full periods of the (tensor, slot) rotation."""
     import math
     return max(warmup, 2 * math.lcm(nslot, nbuf), 48)
 
 
-def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0, check="exact"):
+def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0, check="exact", staged=False, fit_region=False):
     """`steps` timed calls after `warmup` untimed ones (never fewer than two turns of every rotating tensor and
     ring slot, so no buffer is touched for the first time inside the clock), then an optional long run, then a
-    pass of the same steps with the dispatch timestamps of every kernel launch."""
+    pass of the same steps with the dispatch timestamps of every kernel launch.  With `staged` the peer's payload
+    is handed to the emulated wire before every call instead of sitting in the receive slots beforehand."""
     n = N_PREFILL
     for k in TUNING_KEYS:
         os.environ.pop(k, None)
@@ -90,23 +112,39 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     fn = tbv.raw_fn()
     ps = ctypes.c_void_p(st.cuda_stream)
     ptrs = [(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(o.data_ptr())) for x, o in zip(locs, outs)]
-    tbv.peer_resident(b)               # the peer's payload sits in every receive slot before the clock starts
+    if not staged:
+        tbv.peer_resident(b)           # the peer's payload sits in every receive slot before the clock starts
+    stage, pb = tbv.lib().tbv_emu_stage_peer, ctypes.c_void_p(b.data_ptr())
     counter = [0]
 
     def step():
         pa, po = ptrs[counter[0] % nbuf]
         counter[0] += 1
+        if staged and stage(pb, n) != 0:
+            raise RuntimeError("tbv_emu_stage_peer failed")
         rc = fn(pa, po, n, 2, ps)
         if rc != 0:
             raise RuntimeError(f"tbv_ar_allreduce rc={rc}")
 
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev_us = [None]
+
     def timed(k):
+        """Host clock around exactly k steps between two device-wide synchronisations.  Inside the region two events on
+        the caller's stream bracket the launches after the first (the first one's start-up, the host's launch latency
+        on a drained stream, is not a launch duration): device time / (k - 1) is the average launch."""
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(k):
-            step()
+        step()
+        if k > 1:
+            ev[0].record(st)
+            for _ in range(k - 1):
+                step()
+            ev[1].record(st)
         torch.cuda.synchronize()
-        return time.perf_counter() - t0
+        dt = time.perf_counter() - t0
+        ev_us[0] = ev[0].elapsed_time(ev[1]) * 1e3 / (k - 1) if k > 1 else None
+        return dt
 
     for _ in range(own_warmup(warmup, nslot, nbuf)):
         step()
@@ -117,22 +155,19 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
         timed(min(steps, 48))
     tbv.stats4()                       # drop what the warm-up (and the first call's stream probe) accumulated
     wall = timed(steps)
+    ev_timed_us = ev_us[0]
     tbv.stats4()
+    # what the region costs beside its steps: a second region of twice the steps gives slope and intercept
+    region = None
+    if fit_region and steps <= 500:
+        w2 = min(timed(2 * steps) for _ in range(3))
+        w1 = min([wall] + [timed(steps) for _ in range(2)])
+        region = {"steps_1x_us": round(w1 * 1e6, 2), "steps_2x_us": round(w2 * 1e6, 2), "per_step_us": round((w2 - w1) / steps * 1e6, 3),
+                  "fixed_us": round((2 * w1 - w2) * 1e6, 2),
+                  "what": "best of three host-clocked regions of K and of 2K steps: per_step = (T(2K) - T(K)) / K is the steady step, fixed = "
+                          "2 T(K) - T(2K) is what one region pays for starting on a drained stream and for seeing the end of the last kernel"}
     long_wall = timed(long_steps) if long_steps else None
-
-    def evented(k):
-        """The same region again with one event before and one after it on the caller's stream: device time per launch."""
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record(st)
-        for _ in range(k):
-            step()
-        e1.record(st)
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / k
-
-    ev_us = evented(steps)
-    ev_long_us = evented(long_steps) if long_steps else None
+    ev_long_us = ev_us[0] if long_steps else None
     # host cost of one call, from a burst short enough never to wait for room in the ring
     torch.cuda.synchronize()
     tbv.stats4()
@@ -167,7 +202,7 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     for k, _ in env:
         os.environ.pop(k, None)
     return {"wall": wall, "steps": steps, "long_wall": long_wall, "long_steps": long_steps, "ok": ok and not err, "enq_us": enq,
-            "ev_us": ev_us, "ev_long_us": ev_long_us,
+            "ev_us": ev_timed_us, "ev_long_us": ev_long_us, "region": region,
             "pack_us": pack_us, "pack_min_us": pack_min, "n_pack": n_pack, "sum_us": sum_us, "sum_min_us": sum_min, "n_sum": n_sum}
 
 
@@ -194,6 +229,11 @@ def run_achievable(tbv):
         out[name] = {"GBps": round(mult * nbytes / (mean * 1e-6) / 1e9, 1), "avg_us": round(mean, 2), "min_us": round(mn, 2),
                      "frac_of_peak": round(mult * nbytes / (mean * 1e-6) / HBM_PEAK, 4)}
     out["empty_kernel_launch_to_launch_us"] = round(tbv.launch_floor(2000), 2)
+    fl = tbv.step_floor(N_PREFILL, 480)
+    out["step_floor_16MiB_cold"] = {"us": round(fl, 2), "GBps_4N": round(4 * N_PREFILL / (fl * 1e-6) / 1e9, 1),
+                                    "what": "a kernel that only moves the step's four streams (reads local and received, writes the uncached bounce and "
+                                            "the bf16 sum; no counting, no completion word, no gate) on the same cache-cold rotation: no form of the "
+                                            "step can be shorter than this"}
     return out
 
 
@@ -377,6 +417,45 @@ def run_rmsnorm_fusion(tbv, torch, synth, st):
     return out
 
 
+def run_codec_accuracy(tbv, torch, synth, st):
+    """The codec's own accuracy metric: relative L2 error and SNR of the coded all-reduce (through the library, 2 MiB
+    bf16 calls with TBV_CODEC=1) against the exact sum of the two operands, whole-tensor and on the non-outlier elements,
+    on the prefill distribution with and without its 0.1 % outliers, on N(0,1) and on U[-4,4]."""
+    from libtbvcoll_amd import codec_metric
+    numel = 1 << 20
+    for k in TUNING_KEYS:
+        os.environ.pop(k, None)
+    os.environ["TBV_NSLOT"] = "4"
+    os.environ["TBV_CODEC"] = "1"
+    tbv.shutdown()
+    tbv.init(0, "rail0,rail1", "", cap_bytes=2 * numel)
+    out = {"what": "relative L2 error (and SNR) of out = decode(own image) + decode(peer image) against float64(a) + float64(b); "
+                   "`typical` = over the elements that are not outliers (|x| < cut in both operands); stretched groups = groups of 128 of "
+                   "either operand that hold an outlier; rel_l2_uncoded = the same figure for the plain bf16 all-reduce; 2^20 bf16 elements",
+           "group": 128, "code_bits": 8}
+    with torch.cuda.stream(st):
+        for name, gen, cut in codec_metric.distributions(synth):
+            a = torch.from_numpy(gen(100, numel)).to(torch.bfloat16).cuda()
+            b = torch.from_numpy(gen(101, numel)).to(torch.bfloat16).cuda()
+            o = torch.empty_like(a)
+            tbv.stage_peer(b)
+            if not tbv.all_reduce(a, o):
+                raise RuntimeError("coded call not handled")
+            torch.cuda.synchronize()
+            m = codec_metric.accuracy(o.float().cpu().numpy(), a.float().cpu().numpy(), b.float().cpu().numpy(), cut, (a + b).float().cpu().numpy())
+            m["outlier_cut"] = cut
+            out[name] = m
+    ok = not tbv.err()
+    tbv.shutdown()
+    for k in ("TBV_NSLOT", "TBV_CODEC"):
+        os.environ.pop(k, None)
+    out["no_transfer_error"] = ok
+    out["reading"] = ("without outliers the coded sum is within 0.4-0.6 % of the exact one (44-48 dB; plain bf16: 0.18 %); one element in a "
+                      "thousand at +-8 stretches a fifth of the groups and the error on the other elements is about 16 % (16 dB), while "
+                      "the whole-tensor figure still reads 1.3 % because the outliers carry the norm")
+    return out
+
+
 def run_cpu_baseline(torch, synth):
     """The oracle's restatement of the same step (memcpy pack + fp32-upcast sum, RNE) on the host cores."""
     from oracle import oracle
@@ -390,7 +469,8 @@ def run_cpu_baseline(torch, synth):
     da = oracle.torch_bits(torch.from_numpy(synth.normal(0, nd // 2)).to(torch.bfloat16)).copy()
     db = oracle.torch_bits(torch.from_numpy(synth.normal(1, nd // 2)).to(torch.bfloat16)).copy()
     td = oracle.time_reduce_copy(oracle.DT_BF16, da, db, 1, 100, 2000)
-    return {"value": round(5 * n / tn / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+    return {"value": round(5 * n / tn / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port", "host_cpu_count": os.cpu_count(),
+            "host_cpus_usable": len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else None,
             "single_thread_GBps": round(5 * n / t1 / 1e9, 2), "decode_8KB_single_thread_us": round(td * 1e6, 2),
             "sample": f"16 MiB bf16 prefill step (pack 2N + sum 3N), median of 2000 steps on {cores} threads "
                       f"(static contiguous partition) and of 200 steps on 1 thread, about 10 s of CPU work; 8 KB decode step: median of 2000 on 1 thread"}
@@ -402,7 +482,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--decode-iters", type=int, default=10000)
-    ap.add_argument("--legs", default="cold,two,fused,resident,achievable,decode,host,pipeline,codec,rmsnorm,cpu",
+    ap.add_argument("--legs", default="cold,two,fused,staged,resident,achievable,decode,host,pipeline,codec,rmsnorm,cpu",
                     help="comma list of the extra legs to run beside the headline (cold) leg")
     ap.add_argument("--headline-env", default="", help="TBV_X=v,... applied to the headline leg (for profiling one variant)")
     ap.add_argument("--rotate", default=f"{COLD_NSLOT},{COLD_NBUF}",
@@ -436,7 +516,7 @@ def main():
     two_headline = dict(henv).get("TBV_MERGE") == "0" and not fused_headline
     long_steps = 2000 if args.steps < 1000 else 0
     h_nslot, h_nbuf = (int(x) for x in args.rotate.split(","))
-    cold = run_prefill(tbv, torch, synth, st, args.steps, args.warmup, h_nslot, h_nbuf, env=henv, long_steps=long_steps)
+    cold = run_prefill(tbv, torch, synth, st, args.steps, args.warmup, h_nslot, h_nbuf, env=henv, long_steps=long_steps, fit_region=True)
     if args.calibrate_copy:
         src = torch.empty(N_PREFILL, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
@@ -455,26 +535,36 @@ def main():
     ms = cold["wall"] / args.steps * 1e3
     dom_kernel = "sum" if two_headline else ("pack+sum fused" if fused_headline else "pack+sum merged launch")
     dom_bytes = 3 * n if two_headline else alg_step
-    # One launch per step (merged, fused): the launch's duration is the stream's device time over the timed steps divided
-    # by their number, from two events around them.  Timestamps of every single dispatch (a further pass) are reported
-    # beside it: those of back-to-back launches overlap by a varying 0.1-1 us (a dispatch is stamped as started while
-    # its predecessor drains), so their mean reads longer than the step and moves from run to run.
+    # One launch per step (merged, fused): the launch's average duration is measured live inside the timed region, by two
+    # events on the caller's stream around the launches that follow the first one (device time / (steps - 1)).  The
+    # dispatch timestamps of every single launch (a further pass, what rocprofv3's kernel trace averages too) are
+    # reported beside it: a dispatch is stamped as started when its packet is taken up, while its predecessor still
+    # drains, so their mean reads 0.1-0.5 us longer than the step.
+    traffic_kernel = "k_step_sum" if two_headline else ("k_step_pack_sum" if fused_headline else "k_merged")
+    traffic = traffic_from_profile(traffic_kernel)
     if two_headline:
         roof = kernel_roofline(dom_bytes, cold["sum_us"], cold["sum_min_us"], cold["n_sum"], ceiling) or {}
         timing = "dispatch timestamps of every sum launch in a further pass of the same steps"
     else:
-        # with few timed steps the region's device time also holds the first launch's start-up (a few us over 20
-        # launches): the kernel's average is then taken over the long run's 2000 launches, the short region's beside it
-        use_long = bool(cold["ev_long_us"])
-        roof = kernel_roofline(dom_bytes, cold["ev_long_us"] if use_long else cold["ev_us"], cold["sum_min_us"],
-                               cold["long_steps"] if use_long else args.steps, ceiling) or {}
-        roof["timed_steps_avg_launch_us"] = round(cold["ev_us"], 3)
-        roof["per_dispatch_timestamps"] = {"avg_us": round(cold["sum_us"], 3), "min_us": round(cold["sum_min_us"], 3), "launches": cold["n_sum"]}
-        timing = ("two events on the caller's stream around a run of launches, device time / launches: the steps of the host-clocked "
-                  "region run once more right after it (timed_steps_avg_launch_us) and, when those are fewer than 1000, the long "
-                  "run's 2000 (avg_launch_us); per_dispatch_timestamps: start and end stamps of every launch in a further pass")
-    traffic_kernel = "k_step_sum" if two_headline else ("k_step_pack_sum" if fused_headline else "k_merged")
-    traffic = traffic_from_profile(traffic_kernel)
+        roof = kernel_roofline(dom_bytes, cold["ev_us"] or cold["sum_us"], cold["sum_min_us"], max(args.steps - 1, 1), ceiling) or {}
+        roof["per_dispatch_timestamps"] = {"avg_us": round(cold["sum_us"], 3), "min_us": round(cold["sum_min_us"], 3), "launches": cold["n_sum"],
+                                           "frac": round(dom_bytes / (cold["sum_us"] * 1e-6) / HBM_PEAK, 4) if cold["sum_us"] else None}
+        timing = ("avg_launch_us: two events on the caller's stream inside the timed region, around the launches after the first, device "
+                  "time / (steps - 1); per_dispatch_timestamps: start and end stamps of every launch in a further pass (what a kernel "
+                  "trace averages)")
+    roof["denominator"] = ("4N: the local tensor is read once" if fused_headline else "3N (sum kernel alone)" if two_headline else
+                           "5N = pack 2N + sum 3N algorithmic bytes; the sum blocks' read of the local tensor is issued but served by the L2, see frac_fabric")
+    if traffic and roof.get("avg_launch_us"):
+        roof["frac_fabric"] = round(traffic / (roof["avg_launch_us"] * 1e-6) / HBM_PEAK, 4)
+        roof["fabric_GBps"] = round(traffic / (roof["avg_launch_us"] * 1e-6) / 1e9, 1)
+        roof["fabric_denominator"] = "bytes that crossed the fabric per launch by FETCH_SIZE + WRITE_SIZE (4.0 N for the merged launch)"
+        if ceiling:
+            roof["frac_fabric_of_measured_copy_ceiling"] = round(traffic / (roof["avg_launch_us"] * 1e-6) / 1e9 / ceiling, 4)
+    pavg = avg_from_profile(traffic_kernel)
+    if pavg and roof.get("avg_launch_us"):
+        roof["profile_avg_launch_us"] = round(pavg, 3)
+        roof["profile_frac"] = round(dom_bytes / (pavg * 1e-6) / HBM_PEAK, 4)
+        roof["profile_source"] = TRACE_FILE
     line = {
         "metric": "reduce-copy GB/s at 16MB bf16", "value": round(alg_step / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
@@ -486,6 +576,8 @@ def main():
                            ("pack kernel 2N + sum kernel 3N = 5N" if two_headline else
                             "pack 2N + sum 3N = 5N in one launch (pack blocks and sum blocks side by side)"),
                    "frac_of_peak": round(alg_step / (ms * 1e-3) / HBM_PEAK, 4),
+                   "frac_of_peak_is": "value / 8 TB/s by the host clock over the timed region: it carries the region's fixed cost "
+                                      "(region.fixed_us / steps per step) on top of the launch average in roofline.avg_launch_us",
                    "frac_of_measured_copy_ceiling": round(alg_step / (ms * 1e-3) / 1e9 / ceiling, 4) if ceiling else None,
                    "nslot": h_nslot, "rotating_tensors": h_nbuf, "rails": 2, "accumulate": "f32, round to nearest even", "bit_exact_vs_torch_add": cold["ok"],
                    "untimed_warmup_steps": own_warmup(args.warmup, h_nslot, h_nbuf) + 2 * min(args.steps, 48),
@@ -494,12 +586,18 @@ def main():
                          traffic=traffic, traffic_source=(TRAFFIC_FILE if traffic else None),
                          timing=timing),
     }
+    if cold["region"]:
+        line["region"] = cold["region"]
+        line["region"]["steady_value_GBps"] = round(alg_step / (cold["region"]["per_step_us"] * 1e-6) / 1e9, 1)
+        line["region"]["steady_frac_of_peak"] = round(alg_step / (cold["region"]["per_step_us"] * 1e-6) / HBM_PEAK, 4)
     if two_headline:
         line["kernels"] = {"pack": kernel_roofline(2 * n, cold["pack_us"], cold["pack_min_us"], cold["n_pack"], ceiling)}
     if cold["long_wall"]:
         lms = cold["long_wall"] / cold["long_steps"] * 1e3
         line["long_run"] = {"steps": cold["long_steps"], "ms_per_step": round(lms, 5), "value": round(alg_step / (lms * 1e-3) / 1e9, 1),
-                            "unit": "GB/s", "frac_of_peak": round(alg_step / (lms * 1e-3) / HBM_PEAK, 4)}
+                            "unit": "GB/s", "frac_of_peak": round(alg_step / (lms * 1e-3) / HBM_PEAK, 4),
+                            "avg_launch_us": round(cold["ev_long_us"], 3) if cold["ev_long_us"] else None,
+                            "what": "the same leg over 2000 steps in one region (host clock; and the in-region event average)"}
     if ach:
         line["achievable"] = ach
     sub_steps = min(max(args.steps, 500), 2000)
@@ -538,6 +636,38 @@ def main():
 
     if "fused" in legs and not fused_headline:
         leg("fused", leg_fused)
+
+    def leg_staged():
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, staged=True)
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_staged"] = {"what": "the same cache-cold step when the peer's payload is NOT in the receive slot at the call: it is handed to the emulated "
+                                       "wire per call (deposit kernel on a side stream + 64-bit flag after this call's pack completion word); one launch "
+                                       "per call: pack blocks, then sum blocks that poll the flag inside the kernel.  Calls on one stream run one after "
+                                       "the other, so every step pays the whole emulated chain (pack's word seen by the host, deposit launched and run, "
+                                       "arrival seen, flag raised and seen by the waiting kernel) beside its own 5N",
+                               "steps": sub_steps, "ms_per_step": round(rms, 5), "value": round(5 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                               "bit_exact": r["ok"], "host_enqueue_us_per_call": round(r["enq_us"], 2),
+                               "kernel": kernel_roofline(5 * n, r["sum_us"], r["sum_min_us"], r["n_sum"]),
+                               "kernel_note": "the launch's duration includes the time its sum blocks wait for the flag"}
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, env=(("TBV_FORCEGATE", 1),))
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_gated_flag_up"] = {"what": "the staged call's launch (pack blocks + gated sum blocks) with its flag already up when the kernel starts "
+                                              "(TBV_FORCEGATE=1 on the early-peer workload): what the gate's bounded grid costs against the headline's "
+                                              "ungated merged launch",
+                                      "steps": sub_steps, "ms_per_step": round(rms, 5), "value": round(5 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                                      "frac_of_peak": round(5 * n / (rms * 1e-3) / HBM_PEAK, 4), "bit_exact": r["ok"],
+                                      "host_enqueue_us_per_call": round(r["enq_us"], 2),
+                                      "kernel": kernel_roofline(5 * n, r["ev_us"] or r["sum_us"], r["sum_min_us"], sub_steps - 1, ceiling)}
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, env=(("TBV_STAGEDMERGE", 0),), staged=True)
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_staged_three_launches"] = {"what": "cold_staged in the reference's launch sequence: pack kernel, hipStreamWaitValue64, sum kernel (TBV_STAGEDMERGE=0)",
+                                              "steps": sub_steps, "ms_per_step": round(rms, 5), "bit_exact": r["ok"],
+                                              "host_enqueue_us_per_call": round(r["enq_us"], 2),
+                                              "pack": kernel_roofline(2 * n, r["pack_us"], r["pack_min_us"], r["n_pack"]),
+                                              "sum": kernel_roofline(3 * n, r["sum_us"], r["sum_min_us"], r["n_sum"])}
+
+    if "staged" in legs:
+        leg("staged", leg_staged)
 
     def leg_resident():
         r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, 4, 1)
@@ -585,8 +715,13 @@ def main():
                                    "pack": kernel_roofline(n + img, r["pack_us"], r["pack_min_us"], r["n_pack"], ceiling),
                                    "sum": kernel_roofline(n + 2 * img, r["sum_us"], r["sum_min_us"], r["n_sum"], ceiling)}
 
+    def leg_codec_accuracy():
+        line["cold_int8_codec"]["accuracy"] = run_codec_accuracy(tbv, torch, synth, st)
+
     if "codec" in legs:
         leg("codec", leg_codec)
+        if "cold_int8_codec" in line:
+            leg("codec_accuracy", leg_codec_accuracy)
 
     def leg_rmsnorm():
         line["sum_rmsnorm_fusion"] = run_rmsnorm_fusion(tbv, torch, synth, st)

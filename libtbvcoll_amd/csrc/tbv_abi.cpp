@@ -1,11 +1,11 @@
-// The extern "C" surface of libtbvcoll.so (declared in include/tbvcoll.h).
+// The extern "C" surface of libtbvcoll.so (declared in include/tbvcoll.h and include/tbvcoll_emu.h).
 //
 // Part 1 is what the reference's ctypes binding loads (step4/tbvcoll.py:19-30), replacing
 // step4/libtbvcoll.cpp:279-566; part 2 holds this build's additions that are not about the
 // emulated peer itself (those live beside wire_xfer in tbv_peer.cpp).
 #include <algorithm>
 
-#include "../../include/tbvcoll.h"
+#include "../../include/tbvcoll_emu.h"
 #include "tbv_engine.h"
 
 using namespace tbv;

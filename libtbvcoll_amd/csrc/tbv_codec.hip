@@ -17,8 +17,8 @@
 //   sum        out = T(decode(own image) + decode(received image)): each rank decodes its OWN
 //              payload too, so both ranks of a pair compute the same bits
 //
-// One lane per 16-byte input vector (8 elements of a 2-byte type, 4 of fp32); the 16 (32) lanes
-// of a group reduce min and max with xor shuffles; one block per superblock per iteration.
+// One lane per pair of 16-byte input vectors (16 elements of a 2-byte type, 8 of fp32); the 8 (16) lanes
+// of a group reduce min and max with xor shuffles; a block of 256 lanes takes two (one) superblocks per iteration.
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
@@ -81,27 +81,41 @@ template <> struct Vec<2> {
 };
 
 static constexpr unsigned kSbHeader = 128;      // 16 x (scale, mn)
+static constexpr unsigned kCodecBlock = 256;    // lanes per block
 
+// A lane owns two consecutive 16-byte input vectors (16 elements of a 2-byte type, 8 of fp32): the min/max of a
+// group then needs three (four) shuffle steps per 16 (8) elements, and the codes of a 2-byte type leave as one
+// 16-byte store.  A superblock takes 128 (fp32: 256) lanes, so a block of 256 lanes works on two (one) at a time.
 template <int DT>
-__global__ __launch_bounds__(512) void k_quant(StepArgs g)
+__global__ __launch_bounds__(kCodecBlock) void k_quant(StepArgs g)
 {
-    constexpr int EPV = Vec<DT>::EPV;
-    constexpr unsigned LPG = kCodecGroup / EPV;             // lanes per group: 16 or 32
-    const unsigned tid = threadIdx.x;                      // blockDim.x = 2048 / EPV: one superblock per iteration
+    constexpr int EPV = Vec<DT>::EPV, EPL = 2 * EPV;        // elements per vector, per lane
+    constexpr unsigned LPS = kCodecSuper / EPL;             // lanes per superblock: 128 or 256
+    constexpr unsigned LPG = kCodecGroup / EPL;             // lanes per group: 8 or 16
+    constexpr unsigned SPB = kCodecBlock / LPS;             // superblocks per block and iteration: 2 or 1
+    const unsigned tid = threadIdx.x, lt = tid % LPS;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
     if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
     const size_t nvec = g.nbytes >> 4;
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
     unsigned char* image = (unsigned char*)g.bounce;
-    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
-        const size_t i = sb * blockDim.x + tid;
-        const bool have = i < nvec;
-        float f[EPV];
+    for (size_t sb = (size_t)blockIdx.x * SPB + tid / LPS; sb < nsb; sb += (size_t)gridDim.x * SPB) {
+        const size_t i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
+        const bool have0 = i < nvec, have1 = i + 1 < nvec;
+        float f[EPL];
         float mn = __builtin_inff(), mx = -__builtin_inff();
-        if (have) {
-            Vec<DT>::unpack(g.a[i], f);
+        u32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+        if (have0) v0 = g.a[i];
+        if (have1) v1 = g.a[i + 1];
+        Vec<DT>::unpack(v0, f);
+        Vec<DT>::unpack(v1, f + EPV);
+        if (have0) {
 #pragma unroll
             for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+        }
+        if (have1) {
+#pragma unroll
+            for (int e = EPV; e < EPL; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
         }
 #pragma unroll
         for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
@@ -115,60 +129,67 @@ __global__ __launch_bounds__(512) void k_quant(StepArgs g)
         const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
         if (!group_has) mn = 0.0f;
         unsigned char* sbp = image + sb * kCodecSuperBytes;
-        if ((tid % LPG) == 0) {
+        if ((lt % LPG) == 0) {
             f32x2 hdr = {scale, mn};
-            *(f32x2*)(sbp + (tid / LPG) * 8) = hdr;
+            *(f32x2*)(sbp + (lt / LPG) * 8) = hdr;
         }
-        uint32_t lo = 0, hi = 0;
-        if (have) {
+        uint32_t c[EPL / 4];
 #pragma unroll
-            for (int e = 0; e < EPV; e++) {
-                float t = __builtin_rintf((f[e] - mn) * inv);
-                t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
-                const uint32_t q = (uint32_t)t;
-                if (e < 4) lo |= q << (8 * e); else hi |= q << (8 * (e - 4));
-            }
+        for (int k = 0; k < EPL / 4; k++) c[k] = 0;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            const bool have = e < EPV ? have0 : have1;
+            float t = __builtin_rintf((f[e] - mn) * inv);
+            t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
+            const uint32_t q = have ? (uint32_t)t : 0u;
+            c[e / 4] |= q << (8 * (e % 4));
         }
-        if (EPV == 8) { uint2 c = {lo, hi}; *(uint2*)(sbp + kSbHeader + (size_t)tid * 8) = c; }
-        else *(uint32_t*)(sbp + kSbHeader + (size_t)tid * 4) = lo;
+        unsigned char* cp = sbp + kSbHeader + (size_t)lt * EPL;
+        if (EPL == 16) { u32x4 cv = {c[0], c[1], c[2 % (EPL / 4)], c[3 % (EPL / 4)]}; st_bounce<true>((u32x4*)cp, cv); }
+        else { uint2 cv = {c[0], c[1]}; *(uint2*)cp = cv; }
     }
     if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
 }
 
-__device__ __forceinline__ void decode(const unsigned char* sbp, unsigned tid, unsigned lpg, int epv, float* r)
+// The EPL elements of lane `lt` of one superblock image, decoded.
+template <int EPL>
+__device__ __forceinline__ void decode(const unsigned char* sbp, unsigned lt, unsigned lpg, float* r)
 {
-    const f32x2 hdr = *(const f32x2*)(sbp + (tid / lpg) * 8);
-    uint32_t lo, hi = 0;
-    if (epv == 8) { const uint2 c = *(const uint2*)(sbp + kSbHeader + (size_t)tid * 8); lo = c.x; hi = c.y; }
-    else lo = *(const uint32_t*)(sbp + kSbHeader + (size_t)tid * 4);
-    for (int e = 0; e < epv; e++) {
-        const uint32_t q = ((e < 4 ? lo >> (8 * e) : hi >> (8 * (e - 4))) & 0xffu);
+    const f32x2 hdr = *(const f32x2*)(sbp + (lt / lpg) * 8);
+    uint32_t c[EPL / 4];
+    const unsigned char* cp = sbp + kSbHeader + (size_t)lt * EPL;
+    if (EPL == 16) { const u32x4 cv = *(const u32x4*)cp; c[0] = cv.x; c[1] = cv.y; c[2 % (EPL / 4)] = cv.z; c[3 % (EPL / 4)] = cv.w; }
+    else { const uint2 cv = *(const uint2*)cp; c[0] = cv.x; c[1] = cv.y; }
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        const uint32_t q = (c[e / 4] >> (8 * (e % 4))) & 0xffu;
         r[e] = __builtin_fmaf((float)q, hdr.x, hdr.y);
     }
 }
 
 // out = T(decode(own image) + decode(received image)); g.a = own image, g.b = received image
 template <int DT>
-__global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
+__global__ __launch_bounds__(kCodecBlock) void k_sum_quant(StepArgs g)
 {
-    constexpr int EPV = Vec<DT>::EPV;
-    constexpr unsigned LPG = kCodecGroup / EPV;
-    const unsigned tid = threadIdx.x;
+    constexpr int EPV = Vec<DT>::EPV, EPL = 2 * EPV;
+    constexpr unsigned LPS = kCodecSuper / EPL, LPG = kCodecGroup / EPL, SPB = kCodecBlock / LPS;
+    const unsigned tid = threadIdx.x, lt = tid % LPS;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
     if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     const size_t nvec = g.nbytes >> 4;
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
     const unsigned char* ia = (const unsigned char*)g.a;
     const unsigned char* ib = (const unsigned char*)g.b;
-    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
-        const size_t i = sb * blockDim.x + tid;
+    for (size_t sb = (size_t)blockIdx.x * SPB + tid / LPS; sb < nsb; sb += (size_t)gridDim.x * SPB) {
+        const size_t i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
         if (i >= nvec) continue;
-        float x[EPV], y[EPV];
-        decode(ia + sb * kCodecSuperBytes, tid, LPG, EPV, x);
-        decode(ib + sb * kCodecSuperBytes, tid, LPG, EPV, y);
+        float x[EPL], y[EPL];
+        decode<EPL>(ia + sb * kCodecSuperBytes, lt, LPG, x);
+        decode<EPL>(ib + sb * kCodecSuperBytes, lt, LPG, y);
 #pragma unroll
-        for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
+        for (int e = 0; e < EPL; e++) x[e] = x[e] + y[e];
         __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + i);
+        if (i + 1 < nvec) __builtin_nontemporal_store(Vec<DT>::pack(x + EPV), g.out + i + 1);
     }
     if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
@@ -183,14 +204,19 @@ hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const
     return hipGetLastError();
 }
 
+int g_codec_grid_cap = 2048;
+
 int codec_grid(size_t nbytes, int dtype, bool gated)
 {
     const size_t epv = dtype == 0 ? 4 : 8, nsb = ((nbytes >> 4) * epv + kCodecSuper - 1) / kCodecSuper;
-    const size_t cap = gated ? 256 : 2048;
-    return (int)(nsb < 1 ? 1 : nsb < cap ? nsb : cap);
+    const size_t spb = dtype == 0 ? 1 : 2, want = (nsb + spb - 1) / spb;        // superblocks per block and iteration
+    const size_t cap = gated ? 256 : (size_t)g_codec_grid_cap;
+    return (int)(want < 1 ? 1 : want < cap ? want : cap);
 }
 
 }  // namespace
+
+void set_codec_grid_cap(int cap) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; }
 
 size_t codec_image_bytes(size_t nbytes, int dtype)
 {
@@ -209,9 +235,9 @@ hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timi
     s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
     const int grid = codec_grid(a.nbytes, dtype, false);
     switch (dtype) {
-        case 0: return launch1(k_quant<0>, grid, 512, st, t, s);
-        case 1: return launch1(k_quant<1>, grid, 256, st, t, s);
-        default: return launch1(k_quant<2>, grid, 256, st, t, s);
+        case 0: return launch1(k_quant<0>, grid, (int)kCodecBlock, st, t, s);
+        case 1: return launch1(k_quant<1>, grid, (int)kCodecBlock, st, t, s);
+        default: return launch1(k_quant<2>, grid, (int)kCodecBlock, st, t, s);
     }
 }
 
@@ -228,9 +254,9 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
     s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
     const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr);
     switch (q.dtype) {
-        case 0: return launch1(k_sum_quant<0>, grid, 512, st, t, s);
-        case 1: return launch1(k_sum_quant<1>, grid, 256, st, t, s);
-        default: return launch1(k_sum_quant<2>, grid, 256, st, t, s);
+        case 0: return launch1(k_sum_quant<0>, grid, (int)kCodecBlock, st, t, s);
+        case 1: return launch1(k_sum_quant<1>, grid, (int)kCodecBlock, st, t, s);
+        default: return launch1(k_sum_quant<2>, grid, (int)kCodecBlock, st, t, s);
     }
 }
 

@@ -54,8 +54,11 @@ static constexpr int kMaxSmallThreads = 1024;
 static constexpr int kMaxGrid = 256 * 8;     // 256 CUs, up to 8 resident blocks each
 // A kernel that waits for the flag inside holds its wave slots while it waits.  Whatever has to
 // run for the flag to come up (another stream's copy, another library's kernel) needs slots too,
-// so a gated grid is kept to an eighth of the GPU's 8192 wave slots; the blocks loop instead.
-static constexpr int kGatedMaxGrid = 256;
+// so the part of a grid that waits is kept to half of the GPU's 8192 wave slots at most (1024 blocks
+// of 4 waves); the blocks loop instead.  Measured with the 16 MiB step and its flag already up
+// (pack blocks + gated sum blocks in one launch, cache-cold): 256 blocks x 4 vectors per lane 18.2 us,
+// 512 x 4 15.4, 512 x 2 14.4, 1024 x 4 14.2, 1024 x 2 13.0 (ungated merged launch: 12.35).
+static constexpr int kGatedMaxGrid = 1024;
 
 // ---------------------------------------------------------------- arithmetic
 
@@ -136,9 +139,11 @@ __device__ __forceinline__ void store_sys(unsigned long long* p, unsigned long l
 static constexpr unsigned kGroup = 32;
 static constexpr unsigned kCtrLine = 16;       // words per counter line (64 bytes)
 
-__device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned long long seq,
+// Returns true in thread 0 of the block that found itself the last one (false everywhere else).
+__device__ __forceinline__ bool grid_complete(unsigned long long* word, unsigned long long seq,
                                               unsigned int* ctr, unsigned int bid, unsigned int nblk, int mode)
 {
+    bool was_last = false;
     if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -168,7 +173,9 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
             if (mode == 0) __hip_atomic_store(word, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             else store_sys(word, seq);
         }
+        was_last = last;
     }
+    return was_last;
 }
 
 // Gate of a kernel on a host-visible word reaching seq.  Only block 0's leader
@@ -178,9 +185,12 @@ __device__ __forceinline__ void grid_complete(unsigned long long* word, unsigned
 // are resident.  Every wait is bounded by a tick count of the constant-rate wall
 // clock (100 MHz on gfx950; the host passes ticks computed from the device's
 // reported rate), so every wave leaves the kernel even if nobody raises the word.
+// `also` (optional) is a device word the polling block waits for as well before it republishes: the pack relay of
+// a launch whose pack blocks must all be done before its sum blocks may store (output aliasing the local tensor).
+// Whoever raises it never waits itself, so this adds no way to deadlock.
 __device__ __forceinline__ void gate_wait_as(unsigned bid, const unsigned long long* flag, unsigned long long seq,
                                              unsigned long long limit, unsigned long long* relay,
-                                             unsigned long long* fp, bool acquire)
+                                             unsigned long long* fp, bool acquire, const unsigned long long* also = nullptr)
 {
     if (threadIdx.x == 0) {
         const unsigned long long t0 = wall_clock64();
@@ -193,6 +203,12 @@ __device__ __forceinline__ void gate_wait_as(unsigned bid, const unsigned long l
                 if (wall_clock64() - t0 > limit) {
                     if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);
                     break;
+                }
+            }
+            if (also) {
+                while (__hip_atomic_load(also, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < seq) {
+                    __builtin_amdgcn_s_sleep(1);
+                    if (wall_clock64() - t0 > limit) break;
                 }
             }
             if (relay) __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -232,6 +248,8 @@ struct StepArgs {
     const u32x4* a; size_t nbytes; unsigned long long seq; unsigned long long* fp; int sigmode;
     unsigned long long* pre_word; unsigned long long pre_seq;
     unsigned pack_blocks;       // merged launch: blocks [0, pack_blocks) pack, the rest sum
+    unsigned long long* pack_relay;   // device word: the pack part stores seq here when its last block is done; the sum part of
+                                      // the same launch waits for it (beside its flag) when the output aliases the local tensor
     int b_uncached;             // the received payload lies in uncached memory: the gate needs no cache invalidation
 };
 

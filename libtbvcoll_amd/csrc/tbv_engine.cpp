@@ -349,6 +349,12 @@ int configure(const char* devs, size_t cap)
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
     G.merge = geti("TBV_MERGE", 1);
     G.merge_max = getz("TBV_MERGEMAX", (size_t)256 << 20);
+    // a call whose peer payload has not arrived yet, above the one-kernel size: pack blocks + gated sum blocks in one launch
+    G.staged_merge = geti("TBV_STAGEDMERGE", 1);
+    G.force_gate = geti("TBV_FORCEGATE", 0);
+    set_gated_tuning(geti("TBV_GATEDGRID", 0), geti("TBV_GATEDUNROLL", 0));
+    set_row_grid_cap(geti("TBV_ROWGRID", 0));
+    set_codec_grid_cap(geti("TBV_CODECGRID", 0));
     G.codec = geti("TBV_CODEC", 0);
     G.codec_min = getz("TBV_CODEC_MIN", (size_t)512 << 10);
     // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
@@ -399,23 +405,40 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
         if (G.gpusig) {
             const bool aligned = !(((uintptr_t)ptr | (uintptr_t)sum_out) & 15);
             const bool plain = sum_out && !G.tag && G.kwait != 1 && !(G.railsum && c->R > 1) && aligned && !c->codec;
-            const bool can_fuse = G.fuse && c->resident && plain && !nm;
+            // in place (the output IS the local tensor), or an output that overlaps it in some other way
+            const bool inplace = sum_out == ptr;
+            const bool overlap = sum_out && (uintptr_t)sum_out < (uintptr_t)ptr + nbytes && (uintptr_t)ptr < (uintptr_t)sum_out + nbytes;
+            // measurement aid (TBV_FORCEGATE=1): an early peer's large calls take the gated one-launch form too, so that
+            // form can be timed with its flag already up when the kernel starts
+            const bool gate_resident = G.force_gate && c->resident && nbytes > G.fusewait_max;
+            const bool fuse_wanted = G.fuse && c->resident && plain && !nm && !gate_resident;
             // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
             // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
-            const bool one_kernel = G.onekernel && !can_fuse && plain && G.can_wait_value && nbytes <= G.fusewait_max &&
+            const bool one_kernel = G.onekernel && !fuse_wanted && plain && G.can_wait_value && nbytes <= G.fusewait_max &&
                                     (nm ? nm->rows <= (unsigned)kRowNormMaxSmallRows : small_call_blocks(nbytes) <= kSmallCallMaxBlocks);
             // Payload already in place and too large for the one-kernel call: pack blocks and sum blocks in one
             // launch (a launch costs about 2.4 us of stream time whatever it does).
             // (up to a size: the two halves share the local tensor through the L2 only while they stay close in time;
             // at 1 GiB the merged launch moves 5.1-5.45 TB/s, two launches 5.6)
-            const bool can_merge = G.merge && !can_fuse && !one_kernel && c->resident && plain && G.packsig == 0 && !nm &&
+            const bool mergeable = G.merge && !fuse_wanted && !one_kernel && c->resident && !gate_resident && plain && G.packsig == 0 && !nm &&
                                    nbytes <= G.merge_max;
+            // Pack blocks and sum blocks read the local tensor independently, so a sum block may store out[i] before
+            // the pack block has read a[i]: an output that overlaps the local tensor cannot take the merged launch.
+            // In place it takes the fused body instead (one lane loads a[i] once and does both stores); any other
+            // overlap gets two launches.
+            const bool can_merge = mergeable && !overlap;
+            const bool can_fuse = fuse_wanted || (mergeable && inplace);
+            // The peer's payload is not there yet and the call is too large for the one-kernel form: still one launch,
+            // pack blocks first, then sum blocks that wait for the flag inside the kernel (instead of pack launch, stream
+            // gate, sum launch).  In place, the sum blocks also wait for the last pack block.
+            const bool staged_one = G.staged_merge && G.merge && (!c->resident || gate_resident) && !one_kernel && plain && G.can_wait_value && G.packsig == 0 &&
+                                    !nm && !hold && nbytes <= G.merge_max && (!overlap || inplace);
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
             // completion word alone and that next kernel raises it first thing.
             const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
-            c->deferred = G.defer && !can_fuse && !can_merge && !one_kernel && !G.tag && G.kwait != 1 && G.can_wait_value &&
+            c->deferred = G.defer && !can_fuse && !can_merge && !one_kernel && !staged_one && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
             pa.pre = take_pending(st);
             // test hook: this call's pack never raises its completion word
@@ -424,10 +447,10 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 pa.cflag = nullptr;
                 c->deferred = false;
                 if (launch_pack(pa, st) != hipSuccess) FAIL("pack kernel launch failed");
-            } else if (one_kernel || can_fuse || can_merge) {
+            } else if (one_kernel || can_fuse || can_merge || staged_one) {
                 SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.b_uncached = (G.uncached & 2) != 0; sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
-                if (one_kernel && !c->resident) {
+                if ((one_kernel && !c->resident) || staged_one) {
                     sa.wait_flag = gflag(c->slot); sa.relay = relay_word(c->slot);
                     sa.spin_limit_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);
                 }
@@ -435,8 +458,11 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 KTimer kt(1);
                 const double tq = nowt();
                 const hipError_t e = one_kernel ? (nm ? launch_row_norm(2, &pa, sa, *nm, st, kt.get()) : launch_small_call(pa, sa, st, kt.get()))
+                                   : staged_one ? launch_pipe(pa, sa, st, kt.get(), relay_word(c->slot) + 1)
                                    : can_fuse ? launch_pack_sum(pa, sa, st, kt.get()) : launch_pack_sum_merged(pa, sa, st, kt.get());
-                if (e != hipSuccess) FAIL("%s launch failed", one_kernel ? "one-kernel call" : "pack+sum kernel");
+                if (e != hipSuccess)
+                    FAIL("%s launch failed: %s (%zu B)", one_kernel ? "one-kernel call" : staged_one ? "pack + gated sum kernel" : "pack+sum kernel",
+                         hipGetErrorName(e), nbytes);
                 G.t_post += nowt() - tq;                       // the launch that carries the sum
                 c->fused = true;
             } else if (hold && !c->codec && G.packsig == 0 && !G.tag && G.kwait != 1 && !(((uintptr_t)ptr) & 15)) {
@@ -518,7 +544,10 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
             if (!pa.pre.word) pa.pre = sa.pre;               // at most one signal is pending at a time: the held pack may hold it already
             sa.pre = PreSignal{};
             if (gate) { sa.wait_flag = gate; sa.relay = relay_word(c.slot); }
-            if (launch_pipe(pa, sa, st, kt.get()) != hipSuccess) FAIL("pipeline kernel launch failed");
+            const hipError_t pe = launch_pipe(pa, sa, st, kt.get());
+            if (pe != hipSuccess)
+                FAIL("pipeline kernel launch failed: %s (pack %p -> %p %zu B seq %llu; sum %p + %p -> %p %zu B seq %llu%s)", hipGetErrorName(pe),
+                     pa.src, pa.dst, pa.nbytes, pa.seq, sa.a, sa.b, sa.out, sa.nbytes, sa.seq, gate ? ", gated" : "");
             return 0;
         }
         if ((c.codec ? launch_sum_quant(sa, st, kt.get())
@@ -559,9 +588,7 @@ int enqueue_wait_sum(const void* ptr, void* outp, int dtype, hipStream_t st, con
         // The flag may already be up when the call is made (the peer was early): the payload is then in
         // place before the sum is even launched and the stream needs no gate at all.
         const bool arrived = G.async && !G.tag && G.kwait != 1 && ld_acq(gflag(c.slot)) >= c.seq;
-        // (a row kernel has one block per row and no grid cap: it may only wait inside when its rows are few)
-        const bool fusewait = G.async && !arrived && (pipe || c.held || c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1 &&
-                              !(nm && nm->rows > (unsigned)kRowNormMaxSmallRows);
+        const bool fusewait = G.async && !arrived && (pipe || c.held || c.deferred || c.nbytes <= G.fusewait_max) && !G.tag && G.kwait != 1;
         if (G.async && !arrived && !fusewait && gate_stream(gflag(c.slot)) != 0) return -1;
         if (G.async && G.tag) {
             if (launch_tagchk((const unsigned long long*)(rb + tag_offset(c.nbytes)), c.seq, dbgwords(), st) != hipSuccess)

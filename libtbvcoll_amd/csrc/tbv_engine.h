@@ -80,6 +80,8 @@ struct Engine {
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     int merge = 1;                            // resident peer: pack and sum blocks in one launch (TBV_MERGE)
     size_t merge_max = (size_t)256 << 20;     // TBV_MERGEMAX: largest payload that takes the merged launch
+    int force_gate = 0;                       // measurement aid: early-peer large calls take the gated one-launch form (TBV_FORCEGATE)
+    int staged_merge = 1;                     // peer not there yet: pack blocks + gated sum blocks in one launch (TBV_STAGEDMERGE)
     int streaming = 0;                        // cache-hint profile of the large kernels (TBV_STREAMING, default by ring size)
     int codec = 0;                            // int8 payload codec for payloads of at least codec_min bytes (TBV_CODEC, off by default)
     size_t codec_min = (size_t)512 << 10;     // TBV_CODEC_MIN

@@ -74,7 +74,12 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& s, hipStream_t st, 
 hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 // One launch of the chunked pipeline: pack `p` (a later chunk; uncached bounce, completion word raised by its own
 // blocks) and sum `s` (an earlier chunk, optionally gated inside on s.wait_flag with s.relay) as two sets of blocks.
-hipError_t launch_pipe(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+// p and s may belong to the same call (one launch for a call whose peer payload has not arrived yet); when s.out then
+// overlaps p.src, `pack_relay` (a device word) must be given: the sum blocks wait for the pack blocks through it.
+hipError_t launch_pipe(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr,
+                       unsigned long long* pack_relay = nullptr);
+// Most blocks, and vectors per lane, of a grid (or the part of one) that waits for a flag inside the kernel.
+void set_gated_tuning(int cap, int unroll);
 // A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
 // blocks of 1024 lanes, one 16-byte vector per lane.
 static constexpr int kSmallCallMaxBlocks = 64;       // 1 MiB; 64 x 16 waves = an eighth of the GPU's wave slots
@@ -98,6 +103,7 @@ struct NormArgs {
 static constexpr int kRowNormMaxVecs = 4096;          // 64 KiB per row: 1024 lanes x 4 vectors
 static constexpr int kRowNormMaxSmallRows = 128;      // one-launch form: every block must be resident while it waits
 bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype);
+void set_row_grid_cap(int cap);                       // most blocks of a row-kernel launch (0 = default)
 // mode 0: normed = rmsnorm(s.a) * weight.   mode 1: out = a + b (s.wait_flag optional), normed = rmsnorm(out) * weight.
 // mode 2: the whole small call in one launch (pack `p`, completion word, flag poll, sum, norm).
 hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& s, const NormArgs& n, hipStream_t st, const Timing* t = nullptr);
@@ -107,6 +113,7 @@ static constexpr unsigned kCodecGroup = 128;
 static constexpr unsigned kCodecSuper = 2048;          // elements per superblock
 static constexpr unsigned kCodecSuperBytes = 2176;     // 16 x 8 header bytes + 2048 code bytes
 size_t codec_image_bytes(size_t nbytes, int dtype);
+void set_codec_grid_cap(int cap);                      // most blocks of a codec launch (0 = default)
 hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum_quant(const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 

@@ -122,24 +122,31 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_merged(StepArgs g)
 
 // ---------------------------------------------------------------- the pipeline step
 //
-// One launch of the chunked pipeline: the pack of a later chunk and the sum of an earlier one, as two sets of
-// blocks with their own arguments.  Blocks [0, P) pack chunk i+depth and raise its completion word; the rest
-// wait for chunk i's flag (block P polls the host word and relays it) and sum it.  The pack blocks have the
-// lower indices, so they are placed first and never wait: a rank always sends before it waits.  Per chunk the
-// caller's thread pays one launch instead of a pack launch, a stream wait and a sum launch (3.5 us of host
-// time instead of 11), which is what bounded the 16-chunk pipeline.
-template <int DT, bool STREAM>
+// Pack blocks and GATED sum blocks in one launch, each set with its own arguments.  Blocks [0, P) pack and raise
+// the pack's completion word; the rest wait for a flag (block P polls the host word and relays it) and sum.  The
+// pack blocks have the lower indices, so they are placed first and never wait: a rank always sends before it waits,
+// so two ranks running this against each other cannot deadlock.  Two uses:
+//   chunked pipeline   pack of chunk i+depth + sum of chunk i: per chunk the caller's thread pays one launch instead of
+//                      a pack launch, a stream wait and a sum launch (3.5 us of host time instead of 11)
+//   one staged call    pack and sum of the SAME call when the peer's payload is not there yet (what two real ranks
+//                      see): one launch instead of pack, stream gate, sum.  When the output aliases the local tensor
+//                      the sum blocks also wait for the last pack block (sm.pack_relay), since a sum block may
+//                      otherwise store out[i] while a pack block has yet to read a[i].
+template <int DT, int UP, int US, bool STREAM>
 __global__ __launch_bounds__(kMaxSmallThreads) void k_pipe(StepArgs pk, StepArgs sm)
 {
     const unsigned tid = threadIdx.x, P = pk.pack_blocks;
     if (pk.pre_word && blockIdx.x == 0 && tid == 0) store_sys(pk.pre_word, pk.pre_seq);
     if (blockIdx.x < P) {
-        step_body<DT, 1, true, false, STREAM>(pk, blockIdx.x, P);
-        if (pk.cflag) grid_complete(pk.cflag, pk.seq, pk.pack_arrive, blockIdx.x, P, pk.sigmode);
+        step_body<DT, UP, true, false, STREAM>(pk, blockIdx.x, P);
+        if (pk.cflag) {
+            const bool last = grid_complete(pk.cflag, pk.seq, pk.pack_arrive, blockIdx.x, P, pk.sigmode);
+            if (last && pk.pack_relay) __hip_atomic_store(pk.pack_relay, pk.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
     } else {
         const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
-        if (sm.wait_flag) gate_wait_as(bid, sm.wait_flag, sm.seq, sm.spin_limit, sm.relay, sm.fp, !sm.b_uncached);
-        step_body<DT, 4, false, true, STREAM>(sm, bid, S);     // few blocks wait: each keeps four loads per operand in flight
+        if (sm.wait_flag) gate_wait_as(bid, sm.wait_flag, sm.seq, sm.spin_limit, sm.relay, sm.fp, !sm.b_uncached, sm.pack_relay);
+        step_body<DT, US, false, true, STREAM>(sm, bid, S);     // few blocks wait: each keeps several loads per operand in flight
         if (sm.done) grid_complete(sm.done, sm.seq, sm.done_arrive, bid, S, 1);
     }
 }
@@ -255,6 +262,8 @@ static int g_grid_cap = 1024;
 static bool g_grid_cap_given = false;   // a cap from the environment applies to every launch shape
 static int g_block = kThreads;
 static bool g_stream = false;   // streaming profile (see the cache hints above)
+static int g_gated_cap = kGatedMaxGrid;     // most blocks of a grid (or part of one) that waits for a flag inside
+static int g_gated_unroll = 2;
 
 struct Geom { int grid, block, unroll; };
 
@@ -296,6 +305,13 @@ static Geom geom_for(size_t nbytes, bool writeback = false, bool merged = false)
 
 int pack_grid(size_t nbytes) { return geom_for(nbytes).grid; }
 int sum_grid(size_t nbytes, int) { return geom_for(nbytes).grid; }
+
+void set_gated_tuning(int cap, int unroll)
+{
+    // a waiting block holds its wave slots: never more than half of the GPU's 8192 (1024 blocks of 4 waves)
+    g_gated_cap = cap >= 1 ? (cap > 1024 ? 1024 : cap) : kGatedMaxGrid;
+    g_gated_unroll = (unroll == 1 || unroll == 2 || unroll == 4) ? unroll : 2;
+}
 
 void set_tuning(int unroll, int grid_cap, int block, int streaming)
 {
@@ -377,12 +393,12 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
         s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
         s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
         Geom g = geom_for(a.nbytes);
-        if (a.wait_flag && g.grid > kGatedMaxGrid) g.grid = kGatedMaxGrid;
+        if (a.wait_flag && g.grid > g_gated_cap) g.grid = g_gated_cap;
         return launch_step<false, true>(a.dtype, s, g, st, t);
     }
     size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
     int grid = (int)((n + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid; if (grid < 1) grid = 1;
-    if (a.wait_flag && grid > kGatedMaxGrid) grid = kGatedMaxGrid;
+    if (a.wait_flag && grid > g_gated_cap) grid = g_gated_cap;
     switch (a.dtype) {
         case 0: return launch1(k_sum_narrow<0>, grid, kThreads, st, t, a);
         case 1: return launch1(k_sum_narrow<1>, grid, kThreads, st, t, a);
@@ -390,8 +406,18 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
     }
 }
 
-static bool fill_pack_sum(StepArgs& s, const PackArgs& p, const SumArgs& q)
+static bool overlaps(const void* x, size_t nx, const void* y, size_t ny)
 {
+    const uintptr_t a = (uintptr_t)x, b = (uintptr_t)y;
+    return a < b + ny && b < a + nx;
+}
+
+// `two_readers`: pack and sum are done by different blocks, each reading the local tensor itself; then the output must
+// not overlap the local tensor (a sum block could store out[i] before the pack block has read a[i]).  With one reader
+// (the fused body: one lane loads a[i] once and does both stores) an output equal to the local tensor is fine.
+static bool fill_pack_sum(StepArgs& s, const PackArgs& p, const SumArgs& q, bool two_readers = false)
+{
+    if (two_readers && overlaps(q.out, q.nbytes, p.src, p.nbytes)) return false;
     if (!(al16(p.src) && al16(p.dst) && al16(q.out) && al16(q.b)) || p.src != q.a || p.nbytes != q.nbytes || !p.dst || !q.out || !q.b)
         return false;
     if (q.dtype < 0 || q.dtype > 2 || (q.done && !q.done_arrive) || (p.cflag && !p.arrive)) return false;
@@ -424,7 +450,7 @@ static hipError_t launch_merged_u(const StepArgs& s, int grid, int block, int un
 hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
 {
     StepArgs s{};
-    if (!fill_pack_sum(s, p, q) || p.sigmode != 0) return hipErrorInvalidValue;
+    if (!fill_pack_sum(s, p, q, true) || p.sigmode != 0) return hipErrorInvalidValue;
     const Geom g = geom_for(p.nbytes, false, true);
     s.pack_blocks = (unsigned)g.grid;
     const int grid = 2 * g.grid, u = g.unroll == 8 ? 4 : g.unroll;
@@ -450,37 +476,64 @@ static hipError_t launch2(void (*kernel)(A, B), int grid, int block, hipStream_t
     return hipGetLastError();
 }
 
-hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+template <int DT, bool STREAM>
+static hipError_t launch_pipe_u(int up, int us, int grid, int block, hipStream_t st, const Timing* t, const StepArgs& pk, const StepArgs& sm)
+{
+    if (up == 2) {
+        switch (us) {
+            case 1: return launch2(k_pipe<DT, 2, 1, STREAM>, grid, block, st, t, pk, sm);
+            case 2: return launch2(k_pipe<DT, 2, 2, STREAM>, grid, block, st, t, pk, sm);
+            default: return launch2(k_pipe<DT, 2, 4, STREAM>, grid, block, st, t, pk, sm);
+        }
+    }
+    switch (us) {
+        case 1: return launch2(k_pipe<DT, 1, 1, STREAM>, grid, block, st, t, pk, sm);
+        case 2: return launch2(k_pipe<DT, 1, 2, STREAM>, grid, block, st, t, pk, sm);
+        default: return launch2(k_pipe<DT, 1, 4, STREAM>, grid, block, st, t, pk, sm);
+    }
+}
+
+hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t, unsigned long long* pack_relay)
 {
     if (!p.dst || !p.src || !p.cflag || !p.arrive || p.sigmode != 0 || p.tagp || !al16(p.dst) || !al16(p.src)) return hipErrorInvalidValue;
     if (!q.out || !q.a || !q.b || !al16(q.out) || !al16(q.a) || !al16(q.b) || q.dtype < 0 || q.dtype > 2 || (q.done && !q.done_arrive) ||
         (q.wait_flag && !q.relay))
         return hipErrorInvalidValue;
+    // The two parts read and write at the same time.  Different chunks of one tensor never overlap; pack and sum of the
+    // same bytes do when the call is in place, and are then ordered through the pack relay (which needs the gate's poll).
+    const bool same = overlaps(q.out, q.nbytes, p.src, p.nbytes);
+    if (same && !(pack_relay && q.wait_flag)) return hipErrorInvalidValue;
     StepArgs pk{}, sm{};
     pk.bounce = (u32x4*)p.dst; pk.cflag = p.cflag; pk.pack_arrive = p.arrive; pk.a = (const u32x4*)p.src; pk.nbytes = p.nbytes;
     pk.seq = p.seq; pk.sigmode = p.sigmode; pk.pre_word = p.pre.word; pk.pre_seq = p.pre.seq;
     sm.out = (u32x4*)q.out; sm.a = (const u32x4*)q.a; sm.b = (const u32x4*)q.b; sm.nbytes = q.nbytes; sm.seq = q.seq; sm.fp = q.fp;
     sm.wait_flag = q.wait_flag; sm.relay = q.relay; sm.spin_limit = q.spin_limit_ticks; sm.done = q.done; sm.done_arrive = q.done_arrive;
     sm.b_uncached = q.b_uncached;
+    if (same) { pk.pack_relay = pack_relay; sm.pack_relay = pack_relay; }
     // one block size for both parts; tiny chunks take the generic size too (their single-block shapes do not mix)
     const int block = g_block;
-    int P = (int)(((p.nbytes >> 4) + block - 1) / block), S = (int)(((q.nbytes >> 4) + block - 1) / block);
+    // pack part: one vector per lane, or two from 8 MiB so that the part stays within 2048 blocks in one pass up to 16 MiB
+    const size_t pvec = p.nbytes >> 4, svec = q.nbytes >> 4;
+    const int up = pvec >= (size_t)2 * block * 1024 ? 2 : 1;
+    const int us = q.wait_flag ? g_gated_unroll : 4;
+    int P = (int)((pvec + (size_t)block * up - 1) / ((size_t)block * up)), S = (int)((svec + (size_t)block * us - 1) / ((size_t)block * us));
     if (P < 1) P = 1;
     if (S < 1) S = 1;
-    if (P > g_grid_cap) P = g_grid_cap;
-    if (S > (q.wait_flag ? kGatedMaxGrid : g_grid_cap)) S = q.wait_flag ? kGatedMaxGrid : g_grid_cap;
+    const int pcap = g_grid_cap_given ? g_grid_cap : 2048;
+    if (P > pcap) P = pcap;
+    if (S > (q.wait_flag ? g_gated_cap : g_grid_cap)) S = q.wait_flag ? g_gated_cap : g_grid_cap;
     pk.pack_blocks = (unsigned)P;
     if (g_stream) {
         switch (q.dtype) {
-            case 0: return launch2(k_pipe<0, true>, P + S, block, st, t, pk, sm);
-            case 1: return launch2(k_pipe<1, true>, P + S, block, st, t, pk, sm);
-            default: return launch2(k_pipe<2, true>, P + S, block, st, t, pk, sm);
+            case 0: return launch_pipe_u<0, true>(up, us, P + S, block, st, t, pk, sm);
+            case 1: return launch_pipe_u<1, true>(up, us, P + S, block, st, t, pk, sm);
+            default: return launch_pipe_u<2, true>(up, us, P + S, block, st, t, pk, sm);
         }
     }
     switch (q.dtype) {
-        case 0: return launch2(k_pipe<0, false>, P + S, block, st, t, pk, sm);
-        case 1: return launch2(k_pipe<1, false>, P + S, block, st, t, pk, sm);
-        default: return launch2(k_pipe<2, false>, P + S, block, st, t, pk, sm);
+        case 0: return launch_pipe_u<0, false>(up, us, P + S, block, st, t, pk, sm);
+        case 1: return launch_pipe_u<1, false>(up, us, P + S, block, st, t, pk, sm);
+        default: return launch_pipe_u<2, false>(up, us, P + S, block, st, t, pk, sm);
     }
 }
 

@@ -49,6 +49,14 @@ unsigned int* scratch_on_current_device()
     return (unsigned int*)sym;
 }
 
+// The address if this device's copy has been looked up already, else null; makes no HIP call beyond hipGetDevice.
+unsigned int* bound_scratch_on_current_device()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    return g_scratch_ptr[dev].load(std::memory_order_acquire);
+}
+
 inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
 }  // namespace
@@ -73,9 +81,21 @@ extern "C" int tbv_step_noalloc(void* out, const void* local, const void* receiv
         return -1;
     }
     if (nbytes == 0) return 0;
-    unsigned int* ctr = scratch_on_current_device();
-    if (!ctr) return -1;
     hipStream_t st = (hipStream_t)stream;
+    unsigned int* ctr = bound_scratch_on_current_device();
+    if (!ctr) {
+        // The look-up below can make the runtime load the code object and set the array up, which is not allowed while
+        // a stream is being captured: the first call on a device has to come before any capture (or tbv_ar_init has).
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            fprintf(stderr, "[tbvcoll] no-alloc step: first call on this device is inside a stream capture; call it once "
+                            "(or tbv_ar_init) on the device before capturing\n");
+            return -1;
+        }
+        (void)hipGetLastError();
+        ctr = scratch_on_current_device();
+    }
+    if (!ctr) return -1;
 
     tbv::PackArgs pa{};
     pa.dst = bounce; pa.src = local; pa.nbytes = nbytes; pa.seq = seq;
@@ -85,9 +105,16 @@ extern "C" int tbv_step_noalloc(void* out, const void* local, const void* receiv
     sa.out = out; sa.a = local; sa.b = received; sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = seq;
     sa.done = done_word; sa.done_arrive = ctr + tbv::kCounterWords;
 
+    // Pack blocks and sum blocks of the one-launch form read `local` independently, so a sum block could store out[i]
+    // before the pack block has read local[i]: in place the step takes the fused body (one lane loads local[i] once and
+    // does both stores); an output that overlaps `local` in any other way gets two launches, one after the other.
+    const uintptr_t lo = (uintptr_t)local, oo = (uintptr_t)out;
+    const bool inplace = out == local, overlap = oo < lo + nbytes && lo < oo + nbytes;
     hipError_t e;
-    if (bounce_uncached && nbytes > 16384) {
+    if (bounce_uncached && nbytes > 16384 && !overlap) {
         e = tbv::launch_pack_sum_merged(pa, sa, st);             // pack blocks and sum blocks in one launch
+    } else if (bounce_uncached && nbytes > 16384 && inplace) {
+        e = tbv::launch_pack_sum(pa, sa, st);                    // one body: load once, store to the bounce and to the output
     } else {
         e = tbv::launch_pack(pa, st);
         if (e == hipSuccess) e = tbv::launch_sum(sa, st);

@@ -8,7 +8,8 @@
 // kernel's result, step4/libtbvcoll.cpp:162-166), x = float(z), s = 1 / sqrt(mean(x^2) + eps),
 // normed = T(x * s) * weight with the product taken in the storage type.
 //
-// One block per row (L = 64..512 lanes).  Lane t of L holds vectors t, t+L, ... of the row in registers, so the
+// One block per row at a time (L = 64..512 lanes; with more rows than blocks a block takes several rows in turn,
+// keeps its part of the weight row in registers and loads the next row while it reduces the current one).  Lane t of L holds vectors t, t+L, ... of the row in registers, so the
 // row is read once; the sum of squares is accumulated with fused multiply-adds in a fixed
 // order (per lane: its vectors in order, elements in order; per wave: xor butterfly 32, 16,
 // 8, 4, 2, 1; per block: the waves' totals in wave order), which makes the result
@@ -92,65 +93,143 @@ template <> struct Row<2> {
     }
 };
 
+// Sum of squares of the block's row from the lanes' partial sums: wave butterfly, one LDS word per wave, the waves'
+// totals added in wave order.  `slot` alternates between rows so that a fast wave's word for the next row cannot
+// overwrite one a slow wave has yet to read (one barrier per row suffices).
+__device__ __forceinline__ float row_total(float ssq, float (*wave_total)[kMaxSmallThreads / 64], int slot, unsigned tid, unsigned lanes)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+    if ((tid & 63) == 0) wave_total[slot][tid >> 6] = ssq;
+    __syncthreads();
+    float total = wave_total[slot][0];
+    for (unsigned w = 1; w < (lanes >> 6); w++) total += wave_total[slot][w];
+    return total;
+}
+
+// MODE 0 / MODE 1.  A block takes rows blockIdx.x, blockIdx.x + gridDim.x, ...: its lanes keep their vectors of the
+// weight row in registers for all of them, and the loads of the next row are issued before the current row is
+// reduced, so the reduction (shuffles, a barrier, a division and a square root) is covered by memory time.
 template <int DT, int VPL, int MODE>
 __global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormArgs nm)
 {
-    __shared__ float wave_total[kMaxSmallThreads / 64];
+    __shared__ float wave_total[2][kMaxSmallThreads / 64];
     const unsigned tid = threadIdx.x, lanes = blockDim.x, hv = nm.row_vecs;
-    const size_t row0 = (size_t)blockIdx.x * hv;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
-    if (MODE == 2 && g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
-
-    u32x4 x[VPL];
+    const u32x4 zero = {0, 0, 0, 0};
+    u32x4 w[VPL], x[VPL], y[VPL];
 #pragma unroll
     for (int v = 0; v < VPL; v++) {
         const unsigned j = tid + (unsigned)v * lanes;
-        const u32x4 zero = {0, 0, 0, 0};
-        x[v] = j < hv ? g.a[row0 + j] : zero;
-        if (MODE == 2 && j < hv) g.bounce[row0 + j] = x[v];
+        w[v] = j < hv ? ((const u32x4*)nm.weight)[j] : zero;
     }
-    if (MODE == 2) {
-        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
-        if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
-    } else if (MODE == 1 && g.wait_flag) {
-        gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
-    }
-    if (MODE >= 1) {
-        // all loads of the received row before the first store: `out` may alias anything, so a load placed after a
-        // store waits for it
-        u32x4 y[VPL];
+    if (MODE == 1 && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
+    unsigned row = blockIdx.x;
+    if (row < nm.rows) {
+        const size_t r0 = (size_t)row * hv;
 #pragma unroll
         for (int v = 0; v < VPL; v++) {
             const unsigned j = tid + (unsigned)v * lanes;
-            const u32x4 zero = {0, 0, 0, 0};
-            y[v] = j < hv ? g.b[row0 + j] : zero;
+            x[v] = j < hv ? g.a[r0 + j] : zero;
+            if (MODE == 1) y[v] = j < hv ? g.b[r0 + j] : zero;
         }
-#pragma unroll
-        for (int v = 0; v < VPL; v++) x[v] = add_vec<DT>(x[v], y[v]);   // lanes past the row: 0 + 0 = +0 in every type
     }
+    int slot = 0;
+    for (; row < nm.rows; row += gridDim.x, slot ^= 1) {
+        const size_t r0 = (size_t)row * hv;
+        const unsigned nrow = row + gridDim.x;
+        u32x4 xn[VPL], yn[VPL];
+        if (nrow < nm.rows) {                                   // the next row's loads go out before this row's stores
+            const size_t n0 = (size_t)nrow * hv;
+#pragma unroll
+            for (int v = 0; v < VPL; v++) {
+                const unsigned j = tid + (unsigned)v * lanes;
+                xn[v] = j < hv ? g.a[n0 + j] : zero;
+                if (MODE == 1) yn[v] = j < hv ? g.b[n0 + j] : zero;
+            }
+        }
+        if (MODE == 1) {
+#pragma unroll
+            for (int v = 0; v < VPL; v++) x[v] = add_vec<DT>(x[v], y[v]);   // lanes past the row: 0 + 0 = +0 in every type
+        }
+        float ssq = 0.0f;
+#pragma unroll
+        for (int v = 0; v < VPL; v++) {
+            const unsigned j = tid + (unsigned)v * lanes;
+            if (MODE == 1 && j < hv) __builtin_nontemporal_store(x[v], g.out + r0 + j);
+            float f[Row<DT>::EPV];
+            Row<DT>::unpack(x[v], f);                            // lanes past the row hold zeros: they add nothing
+#pragma unroll
+            for (int e = 0; e < Row<DT>::EPV; e++) ssq = __builtin_fmaf(f[e], f[e], ssq);
+        }
+        const float total = row_total(ssq, wave_total, slot, tid, lanes);
+        const float s = 1.0f / __builtin_sqrtf(total / (float)((size_t)hv * Row<DT>::EPV) + nm.eps);
+#pragma unroll
+        for (int v = 0; v < VPL; v++) {
+            const unsigned j = tid + (unsigned)v * lanes;
+            if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], w[v], s), (u32x4*)nm.normed + r0 + j);
+        }
+        if (nrow < nm.rows) {
+#pragma unroll
+            for (int v = 0; v < VPL; v++) { x[v] = xn[v]; if (MODE == 1) y[v] = yn[v]; }
+        }
+    }
+    if (MODE == 1 && g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+}
+
+// MODE 2: the whole small call in one launch, one block per row (all resident together): pack the row into the
+// bounce slot, count the blocks and raise the pack's completion word, poll the flag, then sum and normalise.
+template <int DT, int VPL>
+__global__ __launch_bounds__(kMaxSmallThreads) void k_row_call(StepArgs g, NormArgs nm)
+{
+    __shared__ float wave_total[2][kMaxSmallThreads / 64];
+    const unsigned tid = threadIdx.x, lanes = blockDim.x, hv = nm.row_vecs;
+    const size_t row0 = (size_t)blockIdx.x * hv;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    const u32x4 zero = {0, 0, 0, 0};
+    u32x4 x[VPL], w[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {
+        const unsigned j = tid + (unsigned)v * lanes;
+        x[v] = j < hv ? g.a[row0 + j] : zero;
+        if (j < hv) g.bounce[row0 + j] = x[v];
+    }
+    grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {                             // the weight row arrives while the flag is polled
+        const unsigned j = tid + (unsigned)v * lanes;
+        w[v] = j < hv ? ((const u32x4*)nm.weight)[j] : zero;
+    }
+    if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
+    // all loads of the received row before the first store: `out` may alias anything, so a load placed after a
+    // store waits for it
+    u32x4 y[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; v++) {
+        const unsigned j = tid + (unsigned)v * lanes;
+        y[v] = j < hv ? g.b[row0 + j] : zero;
+    }
+#pragma unroll
+    for (int v = 0; v < VPL; v++) x[v] = add_vec<DT>(x[v], y[v]);
     float ssq = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPL; v++) {
         const unsigned j = tid + (unsigned)v * lanes;
-        if (MODE >= 1 && j < hv) __builtin_nontemporal_store(x[v], g.out + row0 + j);
+        if (j < hv) __builtin_nontemporal_store(x[v], g.out + row0 + j);
         float f[Row<DT>::EPV];
-        Row<DT>::unpack(x[v], f);                            // lanes past the row hold zeros: they add nothing
+        Row<DT>::unpack(x[v], f);
 #pragma unroll
         for (int e = 0; e < Row<DT>::EPV; e++) ssq = __builtin_fmaf(f[e], f[e], ssq);
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
-    if ((tid & 63) == 0) wave_total[tid >> 6] = ssq;
-    __syncthreads();
-    float total = wave_total[0];
-    for (unsigned w = 1; w < (lanes >> 6); w++) total += wave_total[w];
+    const float total = row_total(ssq, wave_total, 0, tid, lanes);
     const float s = 1.0f / __builtin_sqrtf(total / (float)((size_t)hv * Row<DT>::EPV) + nm.eps);
 #pragma unroll
     for (int v = 0; v < VPL; v++) {
         const unsigned j = tid + (unsigned)v * lanes;
-        if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], ((const u32x4*)nm.weight)[j], s), (u32x4*)nm.normed + row0 + j);
+        if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], w[v], s), (u32x4*)nm.normed + row0 + j);
     }
-    if (MODE >= 1 && g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
 
 template <typename A, typename B>
@@ -164,11 +243,20 @@ hipError_t launch2(void (*kernel)(A, B), int grid, int block, hipStream_t st, co
 template <int DT, int MODE>
 hipError_t launch_vpl(int vpl, int grid, int block, hipStream_t st, const Timing* t, const StepArgs& s, const NormArgs& n)
 {
+    if (MODE == 2) {
+        switch (vpl) {
+            case 1: return launch2(k_row_call<DT, 1>, grid, block, st, t, s, n);
+            case 2: return launch2(k_row_call<DT, 2>, grid, block, st, t, s, n);
+            case 4: return launch2(k_row_call<DT, 4>, grid, block, st, t, s, n);
+            default: return launch2(k_row_call<DT, 8>, grid, block, st, t, s, n);
+        }
+    }
+    constexpr int M = MODE == 2 ? 1 : MODE;
     switch (vpl) {
-        case 1: return launch2(k_row_norm<DT, 1, MODE>, grid, block, st, t, s, n);
-        case 2: return launch2(k_row_norm<DT, 2, MODE>, grid, block, st, t, s, n);
-        case 4: return launch2(k_row_norm<DT, 4, MODE>, grid, block, st, t, s, n);
-        default: return launch2(k_row_norm<DT, 8, MODE>, grid, block, st, t, s, n);
+        case 1: return launch2(k_row_norm<DT, 1, M>, grid, block, st, t, s, n);
+        case 2: return launch2(k_row_norm<DT, 2, M>, grid, block, st, t, s, n);
+        case 4: return launch2(k_row_norm<DT, 4, M>, grid, block, st, t, s, n);
+        default: return launch2(k_row_norm<DT, 8, M>, grid, block, st, t, s, n);
     }
 }
 
@@ -185,7 +273,14 @@ hipError_t launch_dt(int dtype, int vpl, int grid, int block, hipStream_t st, co
 
 inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
+// Most blocks of a row-kernel launch.  Every block counted by grid_complete needs a place in the counter lines,
+// which hold 8128 blocks; 2048 x 256 lanes is one block per wave-slot group of the GPU.
+int g_row_grid_cap = 2048;
+constexpr int kRowGatedCap = 512;       // a grid that waits for its flag inside: 512 x 4 waves, a quarter of the GPU's wave slots
+
 }  // namespace
+
+void set_row_grid_cap(int cap) { g_row_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; }
 
 bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype)
 {
@@ -217,7 +312,12 @@ hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const 
     int vpl = 1;
     while (vpl < 8 && (nm.row_vecs + vpl - 1) / vpl > 256) vpl *= 2;
     int block = (int)(((nm.row_vecs + vpl - 1) / vpl + 63) / 64 * 64);
-    const int grid = (int)nm.rows;
+    // One block per row up to the cap, beyond it the blocks loop over rows (and overlap one row's reduction with the
+    // next row's loads).  A grid that waits for its flag inside is kept to the gated cap; the one-launch call (mode 2)
+    // has one block per row by construction (its row count is bounded).
+    int cap = g_row_grid_cap;
+    if (mode == 1 && q.wait_flag && cap > kRowGatedCap) cap = kRowGatedCap;
+    const int grid = mode == 2 ? (int)nm.rows : (int)(nm.rows < (unsigned)cap ? nm.rows : (unsigned)cap);
     switch (mode) {
         case 0: return launch_dt<0>(q.dtype, vpl, grid, block, st, t, s, nm);
         case 1: return launch_dt<1>(q.dtype, vpl, grid, block, st, t, s, nm);

@@ -16,7 +16,7 @@
 
 #include <algorithm>
 
-#include "../../include/tbvcoll.h"
+#include "../../include/tbvcoll_emu.h"
 #include "tbv_dma.h"
 
 namespace tbv {

@@ -11,7 +11,7 @@
 #include <algorithm>
 #include <vector>
 
-#include "../../include/tbvcoll.h"
+#include "../../include/tbvcoll_emu.h"
 
 namespace {
 
@@ -50,6 +50,38 @@ __global__ __launch_bounds__(kBlock) void k_stream(const u32x4* __restrict__ src
         if (!LOOP) break;
     }
     if (KIND == 0 && acc.x == 0x12345678u && acc.y == 0x9abcdef0u && acc.z == 0x0fedcba9u) *sink = acc;
+}
+
+// The four streams of one all-reduce step and nothing else: read the local tensor and the received payload, write
+// the bounce and the bf16 sum, two vectors per lane, one pass, no block counting, no completion word, no gate.  What
+// the memory system delivers to this body on cache-cold operands is the floor under every form of the step.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t add_bf16x2(uint32_t x, uint32_t y)
+{
+    f32x2 s;
+    s.x = __uint_as_float(x << 16) + __uint_as_float(y << 16);
+    s.y = __uint_as_float(x & 0xffff0000u) + __uint_as_float(y & 0xffff0000u);
+    bf16x2 r = __builtin_convertvector(s, bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__global__ __launch_bounds__(kBlock) void k_step_floor(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out, size_t nvec)
+{
+    const size_t base = (size_t)blockIdx.x * kBlock * 2;
+    u32x4 x[2], y[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const size_t i = base + (size_t)u * kBlock + threadIdx.x;
+        if (i < nvec) { x[u] = a[i]; y[u] = __builtin_nontemporal_load(b + i); }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const size_t i = base + (size_t)u * kBlock + threadIdx.x;
+        if (i >= nvec) continue;
+        u32x4 r = {add_bf16x2(x[u].x, y[u].x), add_bf16x2(x[u].y, y[u].y), add_bf16x2(x[u].z, y[u].z), add_bf16x2(x[u].w, y[u].w)};
+        __builtin_nontemporal_store(x[u], bounce + i);
+        __builtin_nontemporal_store(r, out + i);
+    }
 }
 
 __global__ void k_nothing(u32x4* sink) { if (sink && threadIdx.x == 4096) sink->x = 1; }
@@ -139,6 +171,54 @@ extern "C" int tbv_emu_hbm_probe(int kind, size_t bytes, size_t pool_bytes, int 
     if (mean_us) *mean_us = sum / reps;
     if (min_us) *min_us = mn;
     return 0;
+}
+
+// Device time per launch of k_step_floor on `bytes` of bf16 (a multiple of 16), `reps` launches back to back between
+// two events, rotating over 12 local/output tensors and 16 received/bounce buffers (beyond the Infinity Cache for
+// 16 MiB).  The bounce buffers are uncached memory, as the library's send ring is; they are kept until the process
+// ends (uncached memory is never handed back to the driver here).
+extern "C" int tbv_emu_step_floor(size_t bytes, int reps, double* us_per_launch)
+{
+    constexpr int NA = 12, NB = 16;
+    static char* bounce_pool = nullptr;
+    static size_t bounce_pool_bytes = 0;
+    if (bytes < 4096 || (bytes & 15) || bytes > ((size_t)64 << 20) || reps < 1 || reps > 100000 || !us_per_launch) return -1;
+    if (bounce_pool_bytes < NB * bytes) {
+        char* p = nullptr;
+        if (hipExtMallocWithFlags((void**)&p, NB * bytes, hipDeviceMallocUncached) != hipSuccess) return -1;
+        bounce_pool = p; bounce_pool_bytes = NB * bytes;     // a smaller, older pool stays allocated on purpose
+    }
+    char *a = nullptr, *o = nullptr, *b = nullptr;
+    hipStream_t st = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = -1;
+    const size_t nvec = bytes >> 4;
+    const dim3 grid((unsigned)((nvec + 2 * kBlock - 1) / (2 * kBlock)));
+    auto run = [&](int i) {
+        hipLaunchKernelGGL(k_step_floor, grid, dim3(kBlock), 0, st, (const u32x4*)(a + (size_t)(i % NA) * bytes), (const u32x4*)(b + (size_t)(i % NB) * bytes),
+                           (u32x4*)(bounce_pool + (size_t)(i % NB) * bytes), (u32x4*)(o + (size_t)(i % NA) * bytes), nvec);
+    };
+    if (hipMalloc((void**)&a, NA * bytes) == hipSuccess && hipMalloc((void**)&o, NA * bytes) == hipSuccess &&
+        hipMalloc((void**)&b, NB * bytes) == hipSuccess && hipMemset(a, 0x3c, NA * bytes) == hipSuccess &&
+        hipMemset(b, 0x3d, NB * bytes) == hipSuccess && hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess &&
+        hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+        for (int i = 0; i < 96; i++) run(i);
+        (void)hipStreamSynchronize(st);
+        (void)hipEventRecord(e0, st);
+        for (int i = 0; i < reps; i++) run(i);
+        (void)hipEventRecord(e1, st);
+        float ms = 0;
+        if (hipStreamSynchronize(st) == hipSuccess && hipGetLastError() == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) {
+            *us_per_launch = ms * 1e3 / reps; rc = 0;
+        }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (st) (void)hipStreamDestroy(st);
+    if (a) (void)hipFree(a);
+    if (o) (void)hipFree(o);
+    if (b) (void)hipFree(b);
+    return rc;
 }
 
 // Launch-to-launch time of an empty kernel in one stream, in microseconds: `reps` launches bracketed by two

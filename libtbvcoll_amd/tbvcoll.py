@@ -33,7 +33,7 @@ _DEFAULT_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtbvco
 _VP, _SZ, _I, _U64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_ulonglong
 _PD, _PU, _PI, _PSZ = (ctypes.POINTER(t) for t in (ctypes.c_double, ctypes.c_ulonglong, ctypes.c_int, ctypes.c_size_t))
 
-# symbol -> (restype, argtypes): everything include/tbvcoll.h declares
+# symbol -> (restype, argtypes): everything include/tbvcoll.h and include/tbvcoll_emu.h declare
 _SIGNATURES = {
     "tbv_ar_init": (_I, [_I, ctypes.c_char_p, ctypes.c_char_p, _I, _SZ]),
     "tbv_ar_allreduce": (_I, [_VP, _VP, _SZ, _I, _VP]),
@@ -55,6 +55,7 @@ _SIGNATURES = {
     "tbv_emu_run_pack": (_I, [_VP, _SZ, _I, _VP]), "tbv_emu_run_sum": (_I, [_VP, _VP, _VP, _SZ, _I, _VP]),
     "tbv_step_noalloc": (_I, [_VP, _VP, _VP, _VP, _I, _SZ, _I, _VP, _VP, _U64, _VP]),
     "tbv_emu_hbm_probe": (_I, [_I, _SZ, _SZ, _I, _PD, _PD]), "tbv_emu_launch_floor": (_I, [_I, _PD]),
+    "tbv_emu_step_floor": (_I, [_SZ, _I, _PD]),
     "tbv_ar_allreduce_rmsnorm": (_I, [_VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
     "tbv_emu_run_sum_norm": (_I, [_I, _VP, _VP, _VP, _VP, _VP, ctypes.c_float, _SZ, _SZ, _I, _VP]),
     "tbv_emu_codec_image_bytes": (_SZ, [_SZ, _I]),
@@ -278,6 +279,15 @@ def launch_floor(reps=2000, so=_DEFAULT_SO):
     return v.value
 
 
+def step_floor(nbytes, reps=480, so=_DEFAULT_SO):
+    """Microseconds per launch of a kernel that only moves the four streams of one bf16 step of `nbytes`
+    (no counting, no signal, no gate) over rotating cache-cold buffers: the floor under every form of the step."""
+    l = _lib or load(so)
+    v = ctypes.c_double()
+    _check(l.tbv_emu_step_floor(nbytes, reps, ctypes.byref(v)), "tbv_emu_step_floor")
+    return v.value
+
+
 def footprints():
     """[wait entered, wait passed, pack started, sum done, wait timed out] sequence numbers (TBV_KWAIT=1)."""
     buf = (ctypes.c_ulonglong * 5)()
@@ -313,10 +323,18 @@ def all_reduce_rmsnorm(t: torch.Tensor, weight: torch.Tensor, eps: float, out: t
     if nb == 0 or nb > _cap:
         return None
     hidden = t.shape[-1]
+    # what the row kernel takes: rows of whole 16-byte vectors, at most 64 KiB each, every buffer 16-byte aligned.
+    # Anything else is declined here (the caller falls back) rather than turned into an error by the library.
+    row_bytes = hidden * t.element_size()
+    if row_bytes % 16 or row_bytes > 65536:
+        return None
+    if normed is not None and (not normed.is_contiguous() or normed.dtype is not t.dtype or normed.numel() != t.numel()):
+        return None
+    ptrs = [t.data_ptr(), weight.data_ptr()] + [x.data_ptr() for x in (out, normed) if x is not None]
+    if any(p % 16 for p in ptrs):
+        return None
     if normed is None:
         normed = torch.empty_like(t)
-    elif not normed.is_contiguous() or normed.dtype is not t.dtype or normed.numel() != t.numel():
-        return None
     rc = _lib.tbv_ar_allreduce_rmsnorm(pin, pout, _VP(normed.data_ptr()), _VP(weight.data_ptr()), eps,
                                        t.numel() // hidden, hidden, code, _stream())
     if rc == -2:

@@ -1,5 +1,5 @@
 /*
- * A plain C caller of the library: includes include/tbvcoll.h as C, links
+ * A plain C caller of the library: includes include/tbvcoll.h (through tbvcoll_emu.h) as C, links
  * libtbvcoll.so, and runs one all-reduce of each dtype code against a host
  * computed sum.  Built by tests/test_c_client.py (compile + link without a
  * GPU; run on the GPU box).  Inputs are small integers, so the sums are exact
@@ -12,7 +12,7 @@
 
 #include <hip/hip_runtime_api.h>
 
-#include "tbvcoll.h"
+#include "tbvcoll_emu.h"      /* the emulated peer (includes tbvcoll.h, the boundary) */
 
 #define CHECK(x) do { if ((x) != hipSuccess) { fprintf(stderr, "HIP call failed at line %d\n", __LINE__); return 2; } } while (0)
 

@@ -10,15 +10,19 @@ import pytest
 from libtbvcoll_amd import tbvcoll
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "tbvcoll.h")
+HEADER = os.path.join(ROOT, "include", "tbvcoll.h")             # the boundary and the entry points added to it
+HEADER_EMU = os.path.join(ROOT, "include", "tbvcoll_emu.h")     # the emulated peer, test hooks, measurement aids
 REFERENCE_SYMBOLS = ["tbv_ar_init", "tbv_ar_allreduce", "tbv_ar_stats", "tbv_ar_stats4", "tbv_ar_stats5", "tbv_ar_cap",
                      "tbv_ar_async", "tbv_ar_err", "tbv_ar_rails", "tbv_ar_hist", "tbv_ar_fini"]
 
 
-def declared_symbols():
-    txt = open(HEADER).read()
-    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
-    return re.findall(r"\b(tbv_(?:ar|emu)_\w+)\s*\(", txt)
+def declared_symbols(header=None):
+    names = []
+    for h in ([header] if header else [HEADER, HEADER_EMU]):
+        txt = open(h).read()
+        txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+        names += re.findall(r"\b(tbv_(?:ar|emu|step)_\w+)\s*\(", txt)
+    return names
 
 
 def test_library_exports_every_declared_symbol():
@@ -28,7 +32,13 @@ def test_library_exports_every_declared_symbol():
     for n in REFERENCE_SYMBOLS:                      # the eleven the reference's binding uses (step4/tbvcoll.py:19-30)
         assert n in names
     for n in names:
-        assert hasattr(lib, n), f"{n} is declared in include/tbvcoll.h but not exported"
+        assert hasattr(lib, n), f"{n} is declared in include/ but not exported"
+    # the boundary header holds no test hook: nothing of the emulated peer is declared there
+    main = declared_symbols(HEADER)
+    assert not [n for n in main if n.startswith("tbv_emu_")], main
+    assert set(REFERENCE_SYMBOLS) <= set(main) and "tbv_step_noalloc" in main
+    # and the Python binding binds exactly what the two headers declare
+    assert set(tbvcoll._SIGNATURES) == set(names)
 
 
 def test_calls_before_init_fail_cleanly():

@@ -187,6 +187,8 @@ MODES = {
     "streaming": {"TBV_STREAMING": 1},
     "streaming_unroll2": {"TBV_STREAMING": 1, "TBV_UNROLL": 2},
     "merge_off": {"TBV_MERGE": 0},
+    "staged_two_launches": {"TBV_STAGEDMERGE": 0},
+    "fusewait_small": {"TBV_FUSEWAIT": 8192},
 }
 
 
@@ -289,7 +291,68 @@ def test_resident_peer_merged_launch_ragged(orc, streaming):
                 assert tbv.all_reduce(c)                               # in place
                 torch.cuda.synchronize()
                 assert first_diff(c, want) is None, (name, numel, "in place")
+                # in place the peer must still be sent the ORIGINAL tensor: no sum block may overwrite a vector
+                # before it has been packed
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), numel * esz, 3) == 0
+                assert np.array_equal(bits_np(img), bits_np(a)), (name, numel, "bounce image of the in-place call")
+                # an output that overlaps the local tensor without being it takes two launches: the image is intact
+                # whatever the (undefined) output holds
+                if numel > 4096:
+                    base = torch.cat([a, a[:64]])
+                    src, dst = base[:numel], base[64:64 + numel]
+                    assert tbv.all_reduce(src, dst)
+                    torch.cuda.synchronize()
+                    assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), numel * esz, 3) == 0
+                    assert np.array_equal(bits_np(img), bits_np(a)), (name, numel, "bounce image of the overlapping call")
             tbv.peer_resident(None)
+        assert not tbv.err()
+
+
+@pytest.mark.parametrize("env", [{}, {"TBV_GATEDGRID": 1024, "TBV_GATEDUNROLL": 2}, {"TBV_STREAMING": 1}, {"TBV_STAGEDMERGE": 0}])
+def test_staged_call_in_one_launch(orc, env):
+    """The peer's payload is not there when the call is made and the call is above the one-kernel size: pack blocks
+    and gated sum blocks share one launch.  Ragged sizes, three dtypes, out of place and in place (the sum blocks
+    then also wait for the last pack block), slots reused back to back; the bounce image must be the original
+    tensor every time, and a 16 MiB call in place must equal the out-of-place result."""
+    hip = ctypes.CDLL("libamdhip64.so.7")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    cap = 16 << 20
+    with session(rails=2, cap=cap, TBV_NSLOT=3, **env) as tbv:
+        for name in ("bf16", "f16", "f32"):
+            dt = DT[name]
+            esz = 4 if name == "f32" else 2
+            sizes = [(1 << 20) // esz + 8, (3 << 20) // esz + 7, (2 << 20) // esz + 3, (5 << 20) // esz - 1] + ([cap // esz] if name == "bf16" else [])
+            for k, numel in enumerate(sizes):
+                a = dev(synth.uniform(171 + k, numel), dt); p = dev(synth.uniform(271 + k, numel), dt)
+                want = oracle_sum(orc, a, p)
+                out = torch.empty_like(a)
+                say("staged one launch", name, numel, env)
+                tbv.stage_peer(p)
+                assert tbv.all_reduce(a, out)
+                torch.cuda.synchronize()
+                assert first_diff(out, want) is None, (name, numel)
+                img = torch.empty_like(a)
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), numel * esz, 3) == 0
+                assert np.array_equal(bits_np(img), bits_np(a))
+                c = a.clone()
+                tbv.stage_peer(p)
+                assert tbv.all_reduce(c)                               # in place
+                torch.cuda.synchronize()
+                assert first_diff(c, want) is None, (name, numel, "in place")
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), numel * esz, 3) == 0
+                assert np.array_equal(bits_np(img), bits_np(a)), (name, numel, "bounce image of the in-place call")
+            # back to back without synchronising: slots and relay words are reused while earlier calls still run
+            numel = (2 << 20) // esz + 16
+            keep = []
+            for k in range(8):
+                a = dev(synth.uniform(400 + k, numel), dt); p = dev(synth.uniform(500 + k, numel), dt)
+                out = a.clone() if k % 2 else torch.empty_like(a)
+                tbv.stage_peer(p)
+                assert tbv.all_reduce(out if k % 2 else a, None if k % 2 else out)
+                keep.append((a, p, out))
+            torch.cuda.synchronize()
+            for a, p, out in keep:
+                assert torch.equal(out, a + p), name
         assert not tbv.err()
 
 

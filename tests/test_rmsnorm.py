@@ -107,7 +107,7 @@ def _gpu_inputs(name, rows, hidden, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["bf16", "f16", "f32"])
-@pytest.mark.parametrize("rows,hidden", [(1, 4096), (3, 64), (17, 5120), (128, 4096), (5, 16384), (2048, 4096)])
+@pytest.mark.parametrize("rows,hidden", [(1, 4096), (3, 64), (17, 5120), (128, 4096), (5, 16384), (2048, 4096), (5000, 512), (4097, 1024)])
 def test_row_kernel_bit_exact_vs_oracle(name, rows, hidden):
     from gpu_util import say
     from libtbvcoll_amd import tbvcoll
@@ -174,8 +174,22 @@ def test_allreduce_rmsnorm_entry_point(mode):
             torch.cuda.synchronize()
             assert np.array_equal(bits(out), want_out) and np.array_equal(bits(normed), want_normed)
         tbv.peer_resident(None)
-        # not taken: over the cap, and a row that is not a multiple of 16 bytes raises
+        # not taken (None: the caller falls back, nothing raised, nothing queued): over the cap, a row that is not a
+        # multiple of 16 bytes, a row over 64 KiB, a view that is not 16-byte aligned
+        seq0 = tbv.seq()
         assert tbv.all_reduce_rmsnorm(torch.zeros(4097, 4096, dtype=torch.bfloat16, device="cuda"), W, 1e-5) is None
-        with pytest.raises(RuntimeError):
-            tbv.all_reduce_rmsnorm(torch.zeros(4, 100, dtype=torch.bfloat16, device="cuda"), torch.ones(100, dtype=torch.bfloat16, device="cuda"), 1e-5)
+        assert tbv.all_reduce_rmsnorm(torch.zeros(4, 100, dtype=torch.bfloat16, device="cuda"), torch.ones(100, dtype=torch.bfloat16, device="cuda"), 1e-5) is None
+        assert tbv.all_reduce_rmsnorm(torch.zeros(2, 40000, dtype=torch.bfloat16, device="cuda"), torch.ones(40000, dtype=torch.bfloat16, device="cuda"), 1e-5) is None
+        odd = torch.zeros(4 * 4096 + 4, dtype=torch.bfloat16, device="cuda")[4:].view(4, 4096)      # 8 bytes past a 16-byte boundary
+        assert odd.data_ptr() % 16 == 8 and tbv.all_reduce_rmsnorm(odd, W, 1e-5) is None
+        assert tbv.seq() == seq0 and not tbv.err()
+        # many rows, gated inside the kernel (the row kernel's blocks loop over rows, so its grid can be capped)
+        dt, code, a, b, w = _gpu_inputs("bf16", 3000, 1024, 950)
+        A, B, W2 = a.cuda(), b.cuda(), w.cuda()
+        want_out, want_normed = oracle.sum_rmsnorm(code, bits(a), bits(b), bits(w), 1024, 1e-5)
+        out = torch.empty_like(A)
+        tbv.stage_peer(B)
+        normed = tbv.all_reduce_rmsnorm(A, W2, 1e-5, out=out)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out), want_out) and np.array_equal(bits(normed), want_normed)
         assert not tbv.err()

@@ -20,7 +20,7 @@ def _hip():
 
 
 @pytest.mark.parametrize("name", ["bf16", "f16", "f32"])
-def test_no_alloc_step_matches_existing_entry_points(name):
+def test_no_alloc_step_matches_existing_entry_points(orc, name):
     hip = _hip()
     dt = DT[name]
     esz = 4 if name == "f32" else 2
@@ -67,6 +67,11 @@ def test_no_alloc_step_matches_existing_entry_points(name):
                                         None, None, seq, st) == 0
             torch.cuda.synchronize()
             assert np.array_equal(bits_np(c), bits_np(out_ref))
+            # in place the bounce must still receive the ORIGINAL tensor (no sum block may run ahead of the pack)
+            assert hip.hipMemcpy(img.data_ptr(), bounce, nbytes, 3) == 0
+            assert np.array_equal(bits_np(img), bits_np(a)), (name, numel, "bounce image of the in-place call")
+            # and the CPU oracle agrees with both entry points
+            assert np.array_equal(bits_np(out), bits_np(orc.sum_torch(a.cpu(), b.cpu()))), (name, numel, "oracle")
         # limits and argument checks: clear errors, nothing launched
         a = dev(synth.normal(1, 64), dt); o = torch.empty_like(a)
         big = (1 << 30) + 16
