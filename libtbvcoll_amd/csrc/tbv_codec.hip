@@ -151,45 +151,97 @@ __global__ __launch_bounds__(kCodecBlock) void k_quant(StepArgs g)
     if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
 }
 
-// The EPL elements of lane `lt` of one superblock image, decoded.
-template <int EPL>
-__device__ __forceinline__ void decode(const unsigned char* sbp, unsigned lt, unsigned lpg, float* r)
+// One vector per lane (16 / 32 lanes per group), one superblock per block and iteration.
+template <int DT>
+__global__ __launch_bounds__(512) void k_quant1(StepArgs g)
 {
-    const f32x2 hdr = *(const f32x2*)(sbp + (lt / lpg) * 8);
-    uint32_t c[EPL / 4];
-    const unsigned char* cp = sbp + kSbHeader + (size_t)lt * EPL;
-    if (EPL == 16) { const u32x4 cv = *(const u32x4*)cp; c[0] = cv.x; c[1] = cv.y; c[2 % (EPL / 4)] = cv.z; c[3 % (EPL / 4)] = cv.w; }
-    else { const uint2 cv = *(const uint2*)cp; c[0] = cv.x; c[1] = cv.y; }
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;             // lanes per group: 16 or 32
+    const unsigned tid = threadIdx.x;                      // blockDim.x = 2048 / EPV: one superblock per iteration
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    const size_t nvec = g.nbytes >> 4;
+    const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
+    unsigned char* image = (unsigned char*)g.bounce;
+    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
+        const size_t i = sb * blockDim.x + tid;
+        const bool have = i < nvec;
+        float f[EPV];
+        float mn = __builtin_inff(), mx = -__builtin_inff();
+        if (have) {
+            Vec<DT>::unpack(g.a[i], f);
 #pragma unroll
-    for (int e = 0; e < EPL; e++) {
-        const uint32_t q = (c[e / 4] >> (8 * (e % 4))) & 0xffu;
+            for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+        }
+#pragma unroll
+        for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
+            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+        }
+        const bool group_has = mn <= mx;                       // false when every lane of the group is past the end
+        mn += 0.0f;                                            // a minimum of -0 is stored as +0, whichever zero the reduction met first
+        const float range = mx - mn;
+        const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
+        const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
+        if (!group_has) mn = 0.0f;
+        unsigned char* sbp = image + sb * kCodecSuperBytes;
+        if ((tid % LPG) == 0) {
+            f32x2 hdr = {scale, mn};
+            *(f32x2*)(sbp + (tid / LPG) * 8) = hdr;
+        }
+        uint32_t lo = 0, hi = 0;
+        if (have) {
+#pragma unroll
+            for (int e = 0; e < EPV; e++) {
+                float t = __builtin_rintf((f[e] - mn) * inv);
+                t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
+                const uint32_t q = (uint32_t)t;
+                if (e < 4) lo |= q << (8 * e); else hi |= q << (8 * (e - 4));
+            }
+        }
+        if (EPV == 8) { uint2 c = {lo, hi}; *(uint2*)(sbp + kSbHeader + (size_t)tid * 8) = c; }
+        else *(uint32_t*)(sbp + kSbHeader + (size_t)tid * 4) = lo;
+    }
+    if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
+}
+
+
+__device__ __forceinline__ void decode1(const unsigned char* sbp, unsigned tid, unsigned lpg, int epv, float* r)
+{
+    const f32x2 hdr = *(const f32x2*)(sbp + (tid / lpg) * 8);
+    uint32_t lo, hi = 0;
+    if (epv == 8) { const uint2 c = *(const uint2*)(sbp + kSbHeader + (size_t)tid * 8); lo = c.x; hi = c.y; }
+    else lo = *(const uint32_t*)(sbp + kSbHeader + (size_t)tid * 4);
+    for (int e = 0; e < epv; e++) {
+        const uint32_t q = ((e < 4 ? lo >> (8 * e) : hi >> (8 * (e - 4))) & 0xffu);
         r[e] = __builtin_fmaf((float)q, hdr.x, hdr.y);
     }
 }
 
-// out = T(decode(own image) + decode(received image)); g.a = own image, g.b = received image
+// out = T(decode(own image) + decode(received image)); g.a = own image, g.b = received image.  One output vector per
+// lane, so every load and store of a wave is one contiguous run (a lane that owns two consecutive vectors would
+// store with a 32-byte stride, which costs this kernel a quarter of its rate); one superblock per block and iteration.
 template <int DT>
-__global__ __launch_bounds__(kCodecBlock) void k_sum_quant(StepArgs g)
+__global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
 {
-    constexpr int EPV = Vec<DT>::EPV, EPL = 2 * EPV;
-    constexpr unsigned LPS = kCodecSuper / EPL, LPG = kCodecGroup / EPL, SPB = kCodecBlock / LPS;
-    const unsigned tid = threadIdx.x, lt = tid % LPS;
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;
+    const unsigned tid = threadIdx.x;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
     if (g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     const size_t nvec = g.nbytes >> 4;
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
     const unsigned char* ia = (const unsigned char*)g.a;
     const unsigned char* ib = (const unsigned char*)g.b;
-    for (size_t sb = (size_t)blockIdx.x * SPB + tid / LPS; sb < nsb; sb += (size_t)gridDim.x * SPB) {
-        const size_t i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
+    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
+        const size_t i = sb * blockDim.x + tid;
         if (i >= nvec) continue;
-        float x[EPL], y[EPL];
-        decode<EPL>(ia + sb * kCodecSuperBytes, lt, LPG, x);
-        decode<EPL>(ib + sb * kCodecSuperBytes, lt, LPG, y);
+        float x[EPV], y[EPV];
+        decode1(ia + sb * kCodecSuperBytes, tid, LPG, EPV, x);
+        decode1(ib + sb * kCodecSuperBytes, tid, LPG, EPV, y);
 #pragma unroll
-        for (int e = 0; e < EPL; e++) x[e] = x[e] + y[e];
+        for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
         __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + i);
-        if (i + 1 < nvec) __builtin_nontemporal_store(Vec<DT>::pack(x + EPV), g.out + i + 1);
     }
     if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
@@ -206,17 +258,20 @@ hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const
 
 int g_codec_grid_cap = 2048;
 
-int codec_grid(size_t nbytes, int dtype, bool gated)
+int g_codec_form = 0;           // quantising kernel: 0 = two vectors per lane, 1 = one vector per lane
+
+// spb = superblocks one block takes per iteration
+int codec_grid(size_t nbytes, int dtype, bool gated, size_t spb)
 {
     const size_t epv = dtype == 0 ? 4 : 8, nsb = ((nbytes >> 4) * epv + kCodecSuper - 1) / kCodecSuper;
-    const size_t spb = dtype == 0 ? 1 : 2, want = (nsb + spb - 1) / spb;        // superblocks per block and iteration
+    const size_t want = (nsb + spb - 1) / spb;
     const size_t cap = gated ? 256 : (size_t)g_codec_grid_cap;
     return (int)(want < 1 ? 1 : want < cap ? want : cap);
 }
 
 }  // namespace
 
-void set_codec_grid_cap(int cap) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; }
+void set_codec_grid_cap(int cap, int form) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; g_codec_form = form == 1 ? 1 : 0; }
 
 size_t codec_image_bytes(size_t nbytes, int dtype)
 {
@@ -233,7 +288,15 @@ hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timi
     s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive;
     s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp; s.sigmode = a.sigmode;
     s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
-    const int grid = codec_grid(a.nbytes, dtype, false);
+    if (g_codec_form == 1) {
+        const int grid1 = codec_grid(a.nbytes, dtype, false, 1);
+        switch (dtype) {
+            case 0: return launch1(k_quant1<0>, grid1, 512, st, t, s);
+            case 1: return launch1(k_quant1<1>, grid1, 256, st, t, s);
+            default: return launch1(k_quant1<2>, grid1, 256, st, t, s);
+        }
+    }
+    const int grid = codec_grid(a.nbytes, dtype, false, dtype == 0 ? 1 : 2);
     switch (dtype) {
         case 0: return launch1(k_quant<0>, grid, (int)kCodecBlock, st, t, s);
         case 1: return launch1(k_quant<1>, grid, (int)kCodecBlock, st, t, s);
@@ -252,11 +315,11 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
     s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks; s.b_uncached = q.b_uncached;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
-    const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr);
+    const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr, 1);
     switch (q.dtype) {
-        case 0: return launch1(k_sum_quant<0>, grid, (int)kCodecBlock, st, t, s);
-        case 1: return launch1(k_sum_quant<1>, grid, (int)kCodecBlock, st, t, s);
-        default: return launch1(k_sum_quant<2>, grid, (int)kCodecBlock, st, t, s);
+        case 0: return launch1(k_sum_quant<0>, grid, 512, st, t, s);
+        case 1: return launch1(k_sum_quant<1>, grid, 256, st, t, s);
+        default: return launch1(k_sum_quant<2>, grid, 256, st, t, s);
     }
 }
 

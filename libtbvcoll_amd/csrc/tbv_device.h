@@ -190,15 +190,19 @@ __device__ __forceinline__ bool grid_complete(unsigned long long* word, unsigned
 // Whoever raises it never waits itself, so this adds no way to deadlock.
 __device__ __forceinline__ void gate_wait_as(unsigned bid, const unsigned long long* flag, unsigned long long seq,
                                              unsigned long long limit, unsigned long long* relay,
-                                             unsigned long long* fp, bool acquire, const unsigned long long* also = nullptr)
+                                             unsigned long long* fp, bool acquire, const unsigned long long* also = nullptr,
+                                             bool relay_may_be_up = false)
 {
     if (threadIdx.x == 0) {
         const unsigned long long t0 = wall_clock64();
         if (bid == 0 || !relay) {
             if (fp && bid == 0) store_sys(fp + FP_WAIT_IN, seq);
             // relaxed polls: an acquire load in the loop would invalidate the caches on every iteration, for this
-            // kernel and for whatever is writing the payload; one acquire fence follows the barrier below
-            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
+            // kernel and for whatever is writing the payload; one acquire fence follows the barrier below.
+            // (relay_may_be_up: a block of the same launch that looked at the flag earlier may have published it already;
+            // one look at device memory then saves the first read of host memory.)
+            const bool up = relay_may_be_up && relay && !also && __hip_atomic_load(relay, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= seq;
+            while (!up && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < seq) {
                 __builtin_amdgcn_s_sleep(1);
                 if (wall_clock64() - t0 > limit) {
                     if (fp) store_sys(fp + FP_WAIT_TIMEOUT, seq);

@@ -354,7 +354,7 @@ int configure(const char* devs, size_t cap)
     G.force_gate = geti("TBV_FORCEGATE", 0);
     set_gated_tuning(geti("TBV_GATEDGRID", 0), geti("TBV_GATEDUNROLL", 0));
     set_row_grid_cap(geti("TBV_ROWGRID", 0));
-    set_codec_grid_cap(geti("TBV_CODECGRID", 0));
+    set_codec_grid_cap(geti("TBV_CODECGRID", 0), geti("TBV_CODECFORM", 0));
     G.codec = geti("TBV_CODEC", 0);
     G.codec_min = getz("TBV_CODEC_MIN", (size_t)512 << 10);
     // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
@@ -411,7 +411,8 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             // measurement aid (TBV_FORCEGATE=1): an early peer's large calls take the gated one-launch form too, so that
             // form can be timed with its flag already up when the kernel starts
             const bool gate_resident = G.force_gate && c->resident && nbytes > G.fusewait_max;
-            const bool fuse_wanted = G.fuse && c->resident && plain && !nm && !gate_resident;
+            const bool in_place_already = c->resident;      // the slot's flag is raised by this rank's own progress thread, never before the call
+            const bool fuse_wanted = G.fuse && in_place_already && plain && !nm && !gate_resident;
             // One launch for a small call: pack, completion word, flag poll and sum in a single kernel whose
             // few blocks are all resident (a decode-size reduction pays one flag wait and one kernel).
             const bool one_kernel = G.onekernel && !fuse_wanted && plain && G.can_wait_value && nbytes <= G.fusewait_max &&
@@ -420,7 +421,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             // launch (a launch costs about 2.4 us of stream time whatever it does).
             // (up to a size: the two halves share the local tensor through the L2 only while they stay close in time;
             // at 1 GiB the merged launch moves 5.1-5.45 TB/s, two launches 5.6)
-            const bool mergeable = G.merge && !fuse_wanted && !one_kernel && c->resident && !gate_resident && plain && G.packsig == 0 && !nm &&
+            const bool mergeable = G.merge && !fuse_wanted && !one_kernel && in_place_already && !gate_resident && plain && G.packsig == 0 && !nm &&
                                    nbytes <= G.merge_max;
             // Pack blocks and sum blocks read the local tensor independently, so a sum block may store out[i] before
             // the pack block has read a[i]: an output that overlaps the local tensor cannot take the merged launch.
@@ -431,7 +432,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             // The peer's payload is not there yet and the call is too large for the one-kernel form: still one launch,
             // pack blocks first, then sum blocks that wait for the flag inside the kernel (instead of pack launch, stream
             // gate, sum launch).  In place, the sum blocks also wait for the last pack block.
-            const bool staged_one = G.staged_merge && G.merge && (!c->resident || gate_resident) && !one_kernel && plain && G.can_wait_value && G.packsig == 0 &&
+            const bool staged_one = G.staged_merge && G.merge && (!in_place_already || gate_resident) && !one_kernel && plain && G.can_wait_value && G.packsig == 0 &&
                                     !nm && !hold && nbytes <= G.merge_max && (!overlap || inplace);
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
@@ -450,6 +451,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             } else if (one_kernel || can_fuse || can_merge || staged_one) {
                 SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.b_uncached = (G.uncached & 2) != 0; sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
+                sa.fp = pa.fp;
                 if ((one_kernel && !c->resident) || staged_one) {
                     sa.wait_flag = gflag(c->slot); sa.relay = relay_word(c->slot);
                     sa.spin_limit_ticks = (unsigned long long)((G.wdog * 2.0 + 1.0) * G.tick_hz);

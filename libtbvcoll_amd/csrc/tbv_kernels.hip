@@ -138,6 +138,14 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_pipe(StepArgs pk, StepArgs
     const unsigned tid = threadIdx.x, P = pk.pack_blocks;
     if (pk.pre_word && blockIdx.x == 0 && tid == 0) store_sys(pk.pre_word, pk.pre_seq);
     if (blockIdx.x < P) {
+        // One look at the flag by the first block's first lane before its own work, without polling: when the peer was
+        // early, the relay word is up before the first sum block is placed (they follow the pack blocks by 2-3 us) and
+        // the gate costs the sum blocks one poll of device memory instead of a read of host memory.  This is a single
+        // load, bounded by memory latency, not a wait for the peer.  (Not with an output that aliases the local
+        // tensor: those sum blocks must see the pack relay first, which only the polling block republishes.)
+        if (blockIdx.x == 0 && tid == 0 && sm.wait_flag && sm.relay && !sm.pack_relay &&
+            __hip_atomic_load(sm.wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= sm.seq)
+            __hip_atomic_store(sm.relay, sm.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         step_body<DT, UP, true, false, STREAM>(pk, blockIdx.x, P);
         if (pk.cflag) {
             const bool last = grid_complete(pk.cflag, pk.seq, pk.pack_arrive, blockIdx.x, P, pk.sigmode);
@@ -145,7 +153,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_pipe(StepArgs pk, StepArgs
         }
     } else {
         const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
-        if (sm.wait_flag) gate_wait_as(bid, sm.wait_flag, sm.seq, sm.spin_limit, sm.relay, sm.fp, !sm.b_uncached, sm.pack_relay);
+        if (sm.wait_flag) gate_wait_as(bid, sm.wait_flag, sm.seq, sm.spin_limit, sm.relay, sm.fp, !sm.b_uncached, sm.pack_relay, true);
         step_body<DT, US, false, true, STREAM>(sm, bid, S);     // few blocks wait: each keeps several loads per operand in flight
         if (sm.done) grid_complete(sm.done, sm.seq, sm.done_arrive, bid, S, 1);
     }

@@ -93,6 +93,9 @@ template <> struct Row<2> {
     }
 };
 
+// A row takes 512 lanes at most (4096 vectors at eight per lane), which leaves the compiler 256 registers per lane.
+static constexpr int kRowMaxLanes = 512;
+
 // Sum of squares of the block's row from the lanes' partial sums: wave butterfly, one LDS word per wave, the waves'
 // totals added in wave order.  `slot` alternates between rows so that a fast wave's word for the next row cannot
 // overwrite one a slow wave has yet to read (one barrier per row suffices).
@@ -107,22 +110,22 @@ __device__ __forceinline__ float row_total(float ssq, float (*wave_total)[kMaxSm
     return total;
 }
 
-// MODE 0 / MODE 1.  A block takes rows blockIdx.x, blockIdx.x + gridDim.x, ...: its lanes keep their vectors of the
-// weight row in registers for all of them, and the loads of the next row are issued before the current row is
-// reduced, so the reduction (shuffles, a barrier, a division and a square root) is covered by memory time.
-template <int DT, int VPL, int MODE>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormArgs nm)
+// MODE 0 / MODE 1.  A block takes rows blockIdx.x, blockIdx.x + gridDim.x, ...  LOOP: the grid has fewer blocks than
+// there are rows; the loads of the next row are then issued before the current row is reduced, so the reduction
+// (shuffles, a barrier, a division and a square root) is covered by memory time.  (The second set of row registers
+// costs occupancy, which is why the one-row form is a variant of its own.)  The weight row is read where it is used,
+// after the reduction: it comes from the L2, and holding it in registers across rows, or asking for it at the start
+// of the kernel (every block wants the same few lines then), measured slower: 2048 x 4096 bf16 cache-cold, 1024
+// looping blocks, 12.58 us against 12.99 (weights first) and 13.27 (weights after the first row's loads); one block
+// per row with the weights read after the reduction: 13.8 us.
+template <int DT, int VPL, int MODE, bool LOOP>
+__global__ __launch_bounds__(kRowMaxLanes) void k_row_norm(StepArgs g, NormArgs nm)
 {
     __shared__ float wave_total[2][kMaxSmallThreads / 64];
     const unsigned tid = threadIdx.x, lanes = blockDim.x, hv = nm.row_vecs;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
     const u32x4 zero = {0, 0, 0, 0};
-    u32x4 w[VPL], x[VPL], y[VPL];
-#pragma unroll
-    for (int v = 0; v < VPL; v++) {
-        const unsigned j = tid + (unsigned)v * lanes;
-        w[v] = j < hv ? ((const u32x4*)nm.weight)[j] : zero;
-    }
+    u32x4 x[VPL], y[VPL];
     if (MODE == 1 && g.wait_flag) gate_wait(g.wait_flag, g.seq, g.spin_limit, g.relay, g.fp, !g.b_uncached);
     unsigned row = blockIdx.x;
     if (row < nm.rows) {
@@ -138,14 +141,17 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormA
     for (; row < nm.rows; row += gridDim.x, slot ^= 1) {
         const size_t r0 = (size_t)row * hv;
         const unsigned nrow = row + gridDim.x;
-        u32x4 xn[VPL], yn[VPL];
-        if (nrow < nm.rows) {                                   // the next row's loads go out before this row's stores
+        // (rows of more than two vectors per lane would spill with a second set of row registers: they load the
+        // next row after the current one's stores instead)
+        constexpr bool PRE = LOOP && VPL <= 2;
+        u32x4 xn[PRE ? VPL : 1], yn[PRE ? VPL : 1];
+        if (PRE && nrow < nm.rows) {                            // the next row's loads go out before this row's stores
             const size_t n0 = (size_t)nrow * hv;
 #pragma unroll
             for (int v = 0; v < VPL; v++) {
                 const unsigned j = tid + (unsigned)v * lanes;
-                xn[v] = j < hv ? g.a[n0 + j] : zero;
-                if (MODE == 1) yn[v] = j < hv ? g.b[n0 + j] : zero;
+                xn[PRE ? v : 0] = j < hv ? g.a[n0 + j] : zero;
+                if (MODE == 1) yn[PRE ? v : 0] = j < hv ? g.b[n0 + j] : zero;
             }
         }
         if (MODE == 1) {
@@ -167,11 +173,17 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_row_norm(StepArgs g, NormA
 #pragma unroll
         for (int v = 0; v < VPL; v++) {
             const unsigned j = tid + (unsigned)v * lanes;
-            if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], w[v], s), (u32x4*)nm.normed + r0 + j);
+            if (j < hv) __builtin_nontemporal_store(Row<DT>::scale(x[v], ((const u32x4*)nm.weight)[j], s), (u32x4*)nm.normed + r0 + j);
         }
+        if (!LOOP) break;
         if (nrow < nm.rows) {
+            const size_t n0 = (size_t)nrow * hv;
 #pragma unroll
-            for (int v = 0; v < VPL; v++) { x[v] = xn[v]; if (MODE == 1) y[v] = yn[v]; }
+            for (int v = 0; v < VPL; v++) {
+                const unsigned j = tid + (unsigned)v * lanes;
+                if (PRE) { x[v] = xn[PRE ? v : 0]; if (MODE == 1) y[v] = yn[PRE ? v : 0]; }
+                else { x[v] = j < hv ? g.a[n0 + j] : zero; if (MODE == 1) y[v] = j < hv ? g.b[n0 + j] : zero; }
+            }
         }
     }
     if (MODE == 1 && g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
@@ -252,12 +264,10 @@ hipError_t launch_vpl(int vpl, int grid, int block, hipStream_t st, const Timing
         }
     }
     constexpr int M = MODE == 2 ? 1 : MODE;
-    switch (vpl) {
-        case 1: return launch2(k_row_norm<DT, 1, M>, grid, block, st, t, s, n);
-        case 2: return launch2(k_row_norm<DT, 2, M>, grid, block, st, t, s, n);
-        case 4: return launch2(k_row_norm<DT, 4, M>, grid, block, st, t, s, n);
-        default: return launch2(k_row_norm<DT, 8, M>, grid, block, st, t, s, n);
-    }
+#define ROWK(V, L) launch2(k_row_norm<DT, V, M, L>, grid, block, st, t, s, n)
+    if ((unsigned)grid < n.rows) return vpl == 1 ? ROWK(1, true) : vpl == 2 ? ROWK(2, true) : vpl == 4 ? ROWK(4, true) : ROWK(8, true);
+    return vpl == 1 ? ROWK(1, false) : vpl == 2 ? ROWK(2, false) : vpl == 4 ? ROWK(4, false) : ROWK(8, false);
+#undef ROWK
 }
 
 template <int MODE>
@@ -273,14 +283,14 @@ hipError_t launch_dt(int dtype, int vpl, int grid, int block, hipStream_t st, co
 
 inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
-// Most blocks of a row-kernel launch.  Every block counted by grid_complete needs a place in the counter lines,
-// which hold 8128 blocks; 2048 x 256 lanes is one block per wave-slot group of the GPU.
-int g_row_grid_cap = 2048;
+// Most blocks of a row-kernel launch: 0 = what is resident at once (see launch_row_norm), else a given number.
+// Every block counted by grid_complete needs a place in the counter lines, which hold 8128 blocks.
+int g_row_grid_cap = 0;
 constexpr int kRowGatedCap = 512;       // a grid that waits for its flag inside: 512 x 4 waves, a quarter of the GPU's wave slots
 
 }  // namespace
 
-void set_row_grid_cap(int cap) { g_row_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; }
+void set_row_grid_cap(int cap) { g_row_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 0; }
 
 bool row_norm_shape_ok(size_t rows, size_t hidden, int dtype)
 {
@@ -312,12 +322,19 @@ hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const 
     int vpl = 1;
     while (vpl < 8 && (nm.row_vecs + vpl - 1) / vpl > 256) vpl *= 2;
     int block = (int)(((nm.row_vecs + vpl - 1) / vpl + 63) / 64 * 64);
+    if (block > kRowMaxLanes) return hipErrorInvalidValue;        // cannot happen for rows within kRowNormMaxVecs
     // One block per row up to the cap, beyond it the blocks loop over rows (and overlap one row's reduction with the
-    // next row's loads).  A grid that waits for its flag inside is kept to the gated cap; the one-launch call (mode 2)
-    // has one block per row by construction (its row count is bounded).
-    int cap = g_row_grid_cap;
+    // next row's loads), every block the same number of rows where that divides.  The cap is what is resident at once
+    // at four waves per SIMD (the looping form's registers allow four to five): 4096 waves.  Measured with 2048 x 4096
+    // bf16, cache-cold: 2048 blocks of one row 13.8 us, 1024 blocks of two rows 13.0, 768 13.4, 512 14.6.  A grid that
+    // waits for its flag inside is kept to half of that; the one-launch call (mode 2) has one block per row by
+    // construction (its row count is bounded).
+    // (the norm-only form needs fewer registers: all 8192 wave slots hold a block of it)
+    int cap = g_row_grid_cap > 0 ? g_row_grid_cap : (mode == 0 ? 8192 : 4096) / (block / 64);
     if (mode == 1 && q.wait_flag && cap > kRowGatedCap) cap = kRowGatedCap;
-    const int grid = mode == 2 ? (int)nm.rows : (int)(nm.rows < (unsigned)cap ? nm.rows : (unsigned)cap);
+    if (cap < 1) cap = 1;
+    const unsigned per_block = (nm.rows + (unsigned)cap - 1) / (unsigned)cap;
+    const int grid = mode == 2 ? (int)nm.rows : (int)((nm.rows + per_block - 1) / per_block);
     switch (mode) {
         case 0: return launch_dt<0>(q.dtype, vpl, grid, block, st, t, s, nm);
         case 1: return launch_dt<1>(q.dtype, vpl, grid, block, st, t, s, nm);

@@ -553,6 +553,58 @@ def test_seeded_mix_of_everything(orc, seed, env):
         assert not tbv.err()
 
 
+def test_gates_inside_kernels_while_another_stream_keeps_the_gpu_busy(orc):
+    """The kernels that wait for their flag inside (the one-kernel decode call, the pack + gated sum launch of a staged
+    large call) hold their wave slots while they wait, and what raises the flag (the emulated peer's deposit kernel on a
+    side stream) needs slots too.  Here a second stream keeps every CU busy with large elementwise kernels while 2000
+    decode calls and 200 staged 1-4 MiB calls run: every result exact, no watchdog, no in-kernel wait that ran into
+    its bound (footprint 4 stays 0; TBV_KWAIT=2 keeps the footprints without the diagnostic wait kernel)."""
+    with session(rails=2, cap=4 << 20, TBV_NSLOT=4, TBV_WDOG=5, TBV_KWAIT=2) as tbv:
+        bg = torch.cuda.Stream()
+        big = torch.ones(64 << 20, dtype=torch.float32, device="cuda")        # 256 MiB: each pass keeps all CUs busy for ~100 us
+        main = torch.cuda.current_stream()
+
+        def load_gpu(n):
+            with torch.cuda.stream(bg):
+                for _ in range(n):
+                    big.mul_(1.0000001)
+
+        load_gpu(50)
+        t0 = time.time()
+        pend, bad = [], 0
+        for it in range(2200):
+            staged_big = it % 11 == 10
+            nb = [1 << 20, 2 << 20, (3 << 20) + 4096, 4 << 20][(it // 11) % 4] + 16 if staged_big else 8192
+            if staged_big and nb > (4 << 20):
+                nb = 4 << 20
+            dt = (torch.bfloat16, torch.float16, torch.float32)[it % 3]
+            numel = nb // (4 if dt == torch.float32 else 2)
+            a = synth.torch_hash_uniform(2 * it + 7, numel).to(dt)
+            p = synth.torch_hash_uniform(2 * it + 8, numel).to(dt)
+            inplace = it % 5 == 0
+            out = a.clone() if inplace else torch.empty_like(a)
+            tbv.stage_peer(p)
+            assert tbv.all_reduce(out if inplace else a, None if inplace else out), it
+            pend.append((it, a, p, out))
+            if it % 8 == 0:
+                load_gpu(4)                                                  # keep the other stream's queue full
+            if len(pend) >= 64:
+                main.synchronize()
+                if tbv.err():
+                    break                                                    # stop at the first failure
+                bad += sum(0 if torch.equal(o, x + y) else 1 for _, x, y, o in pend)
+                pend = []
+        main.synchronize()
+        bad += sum(0 if torch.equal(o, x + y) else 1 for _, x, y, o in pend)
+        say("contention: 2200 calls in", round(time.time() - t0, 2), "s; bad", bad, "footprints", tbv.footprints())
+        torch.cuda.synchronize()
+        assert not tbv.err(), "a watchdog tripped"
+        assert bad == 0
+        assert tbv.footprints()[4] == 0                                      # no in-kernel wait ran into its bound
+        want = oracle_sum(orc, pend[-1][1], pend[-1][2]) if pend else None
+        assert want is None or first_diff(pend[-1][3], want) is None
+
+
 def test_grids_beyond_the_small_counter_groups(orc):
     """Grids of more than 4064 blocks count their completion in groups of 64 instead of 32 (the tuning knobs allow up
     to 8128 blocks): pack, merged launch and sum at that size, staged and early peer, completion words included."""
