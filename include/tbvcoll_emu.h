@@ -107,6 +107,22 @@ void tbv_emu_tag_counts(unsigned long long* checks, unsigned long long* bad_plai
  * never freed), clears the sticky error. */
 void tbv_emu_shutdown(void);
 
+/* ------------------------------------------------------------------ two processes on one GPU
+ *
+ * With TBV_PEER=tcp in the environment of both processes, tbv_ar_init(rank, devs, peer_ip, port, cap) meets a real
+ * peer process instead of emulating one: rank 0 listens on `port`, rank 1 connects to peer_ip:port (retrying for up
+ * to TBV_RDV_TIMEOUT seconds, default 60, while rank 0 is not there yet), per rail the ranks swap and compare what they
+ * must agree on (cap, TBV_NSLOT, rail count, TBV_TAG, TBV_CODEC, TBV_RAIL1MAX, TBV_CHUNK; a mismatch fails both
+ * inits), then one byte each way as a barrier: the shape of the reference's bring-up (step4/libtbvcoll.cpp:371-385,
+ * :403).  Each rail's connection then carries that rail's fragments, through pinned host memory on both sides; the
+ * receive side deposits them into the receive slot and raises the arrival word like the emulated peer.  A two-rank
+ * driver written against the reference (RANK=0/1 processes that call init and all_reduce and nothing else) runs
+ * unchanged.  The tbv_emu_stage_* / tbv_emu_peer_resident calls are refused in this mode.
+ *
+ * tbv_emu_rendezvous runs that rendezvous alone and closes the connections again (sockets only, no GPU; needs
+ * tbv_emu_configure first).  Returns 0, or -1 after a "[tbvcoll] rendezvous: ..." line. */
+int tbv_emu_rendezvous(int rank, const char* peer_ip, int port, double timeout_s);
+
 /* ------------------------------------------------------------------ kernels run alone, for benches and tests */
 
 /* The int8 codec's kernels: the image size of a payload, payload -> image, and two images -> sum. */

@@ -3,10 +3,13 @@
 // Part 1 is what the reference's ctypes binding loads (step4/tbvcoll.py:19-30), replacing
 // step4/libtbvcoll.cpp:279-566; part 2 holds this build's additions that are not about the
 // emulated peer itself (those live beside wire_xfer in tbv_peer.cpp).
+#include <unistd.h>
+
 #include <algorithm>
 
 #include "../../include/tbvcoll_emu.h"
 #include "tbv_engine.h"
+#include "tbv_sock.h"
 
 using namespace tbv;
 
@@ -26,9 +29,8 @@ struct OneCaller {
 
 extern "C" int tbv_ar_init(int rank, const char* devs, const char* peer_ip, int port, size_t cap)
 {
-    (void)peer_ip; (void)port;
     if (G.inited) return 0;
-    const int rc = init_impl(rank, devs, cap);
+    const int rc = init_impl(rank, devs, peer_ip, port, cap);
     if (rc != 0) teardown();               // a failed initialisation leaves nothing allocated and no thread running
     return rc;
 }
@@ -150,6 +152,16 @@ extern "C" int tbv_emu_plan(size_t nbytes, size_t* off, size_t* len)
         if (len) len[r] = l;
     }
     return R;
+}
+
+// The rendezvous of the two-process mode alone (sockets only, no GPU): needs tbv_emu_configure first.
+extern "C" int tbv_emu_rendezvous(int rank, const char* peer_ip, int port, double timeout_s)
+{
+    if (!G.configured || G.inited) return -1;
+    int fds[MAXRAIL];
+    const int rc = sock_rendezvous(rank, peer_ip, port, fds, timeout_s);
+    for (int r = 0; r < MAXRAIL; r++) if (fds[r] >= 0) close(fds[r]);
+    return rc;
 }
 
 extern "C" int tbv_emu_nslot(void) { return G.nslot; }

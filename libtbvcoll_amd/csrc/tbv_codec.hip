@@ -86,142 +86,112 @@ static constexpr unsigned kCodecBlock = 256;    // lanes per block
 // A lane owns two consecutive 16-byte input vectors (16 elements of a 2-byte type, 8 of fp32): the min/max of a
 // group then needs three (four) shuffle steps per 16 (8) elements, and the codes of a 2-byte type leave as one
 // 16-byte store.  A superblock takes 128 (fp32: 256) lanes, so a block of 256 lanes works on two (one) at a time.
-template <int DT>
+template <int DT, int U>
 __global__ __launch_bounds__(kCodecBlock) void k_quant(StepArgs g)
 {
     constexpr int EPV = Vec<DT>::EPV, EPL = 2 * EPV;        // elements per vector, per lane
     constexpr unsigned LPS = kCodecSuper / EPL;             // lanes per superblock: 128 or 256
     constexpr unsigned LPG = kCodecGroup / EPL;             // lanes per group: 8 or 16
-    constexpr unsigned SPB = kCodecBlock / LPS;             // superblocks per block and iteration: 2 or 1
+    constexpr unsigned SPB = kCodecBlock / LPS;             // superblocks per block and pass: 2 or 1
     const unsigned tid = threadIdx.x, lt = tid % LPS;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
     if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
     const size_t nvec = g.nbytes >> 4;
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
+    const size_t stride = (size_t)gridDim.x * SPB;
     unsigned char* image = (unsigned char*)g.bounce;
-    for (size_t sb = (size_t)blockIdx.x * SPB + tid / LPS; sb < nsb; sb += (size_t)gridDim.x * SPB) {
-        const size_t i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
-        const bool have0 = i < nvec, have1 = i + 1 < nvec;
-        float f[EPL];
-        float mn = __builtin_inff(), mx = -__builtin_inff();
-        u32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-        if (have0) v0 = g.a[i];
-        if (have1) v1 = g.a[i + 1];
-        Vec<DT>::unpack(v0, f);
-        Vec<DT>::unpack(v1, f + EPV);
-        if (have0) {
+    // U passes' loads go out together (measured: no gain, see the grid cap's comment)
+    for (size_t sb0 = (size_t)blockIdx.x * SPB + tid / LPS; sb0 < nsb; sb0 += stride * U) {
+        u32x4 v0[U], v1[U];
 #pragma unroll
-            for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
-        }
-        if (have1) {
-#pragma unroll
-            for (int e = EPV; e < EPL; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+        for (int u = 0; u < U; u++) {
+            const size_t sb = sb0 + (size_t)u * stride, i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
+            const u32x4 zero = {0, 0, 0, 0};
+            v0[u] = (sb < nsb && i < nvec) ? g.a[i] : zero;
+            v1[u] = (sb < nsb && i + 1 < nvec) ? g.a[i + 1] : zero;
         }
 #pragma unroll
-        for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
-            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
-            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
-        }
-        const bool group_has = mn <= mx;                       // false when every lane of the group is past the end
-        mn += 0.0f;                                            // a minimum of -0 is stored as +0, whichever zero the reduction met first
-        const float range = mx - mn;
-        const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
-        const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
-        if (!group_has) mn = 0.0f;
-        unsigned char* sbp = image + sb * kCodecSuperBytes;
-        if ((lt % LPG) == 0) {
-            f32x2 hdr = {scale, mn};
-            *(f32x2*)(sbp + (lt / LPG) * 8) = hdr;
-        }
-        uint32_t c[EPL / 4];
+        for (int u = 0; u < U; u++) {
+            const size_t sb = sb0 + (size_t)u * stride;
+            if (sb >= nsb) break;                              // uniform over the wave: a wave lies within one superblock
+            const size_t i = sb * (kCodecSuper / EPV) + (size_t)lt * 2;
+            const bool have0 = i < nvec, have1 = i + 1 < nvec;
+            float f[EPL];
+            float mn = __builtin_inff(), mx = -__builtin_inff();
+            Vec<DT>::unpack(v0[u], f);
+            Vec<DT>::unpack(v1[u], f + EPV);
+            if (have0) {
 #pragma unroll
-        for (int k = 0; k < EPL / 4; k++) c[k] = 0;
+                for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+            }
+            if (have1) {
 #pragma unroll
-        for (int e = 0; e < EPL; e++) {
-            const bool have = e < EPV ? have0 : have1;
-            float t = __builtin_rintf((f[e] - mn) * inv);
-            t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
-            const uint32_t q = have ? (uint32_t)t : 0u;
-            c[e / 4] |= q << (8 * (e % 4));
-        }
-        unsigned char* cp = sbp + kSbHeader + (size_t)lt * EPL;
-        if (EPL == 16) { u32x4 cv = {c[0], c[1], c[2 % (EPL / 4)], c[3 % (EPL / 4)]}; st_bounce<true>((u32x4*)cp, cv); }
-        else { uint2 cv = {c[0], c[1]}; *(uint2*)cp = cv; }
-    }
-    if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
-}
-
-// One vector per lane (16 / 32 lanes per group), one superblock per block and iteration.
-template <int DT>
-__global__ __launch_bounds__(512) void k_quant1(StepArgs g)
-{
-    constexpr int EPV = Vec<DT>::EPV;
-    constexpr unsigned LPG = kCodecGroup / EPV;             // lanes per group: 16 or 32
-    const unsigned tid = threadIdx.x;                      // blockDim.x = 2048 / EPV: one superblock per iteration
-    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
-    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
-    const size_t nvec = g.nbytes >> 4;
-    const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
-    unsigned char* image = (unsigned char*)g.bounce;
-    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
-        const size_t i = sb * blockDim.x + tid;
-        const bool have = i < nvec;
-        float f[EPV];
-        float mn = __builtin_inff(), mx = -__builtin_inff();
-        if (have) {
-            Vec<DT>::unpack(g.a[i], f);
+                for (int e = EPV; e < EPL; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+            }
 #pragma unroll
-            for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
-        }
+            for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
+                mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+                mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+            }
+            const bool group_has = mn <= mx;                       // false when every lane of the group is past the end
+            mn += 0.0f;                                            // a minimum of -0 is stored as +0, whichever zero the reduction met first
+            const float range = mx - mn;
+            const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
+            const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
+            if (!group_has) mn = 0.0f;
+            unsigned char* sbp = image + sb * kCodecSuperBytes;
+            if ((lt % LPG) == 0) {
+                f32x2 hdr = {scale, mn};
+                *(f32x2*)(sbp + (lt / LPG) * 8) = hdr;
+            }
+            uint32_t c[EPL / 4];
 #pragma unroll
-        for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
-            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
-            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
-        }
-        const bool group_has = mn <= mx;                       // false when every lane of the group is past the end
-        mn += 0.0f;                                            // a minimum of -0 is stored as +0, whichever zero the reduction met first
-        const float range = mx - mn;
-        const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
-        const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
-        if (!group_has) mn = 0.0f;
-        unsigned char* sbp = image + sb * kCodecSuperBytes;
-        if ((tid % LPG) == 0) {
-            f32x2 hdr = {scale, mn};
-            *(f32x2*)(sbp + (tid / LPG) * 8) = hdr;
-        }
-        uint32_t lo = 0, hi = 0;
-        if (have) {
+            for (int k = 0; k < EPL / 4; k++) c[k] = 0;
 #pragma unroll
-            for (int e = 0; e < EPV; e++) {
+            for (int e = 0; e < EPL; e++) {
+                const bool have = e < EPV ? have0 : have1;
                 float t = __builtin_rintf((f[e] - mn) * inv);
                 t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), 255.0f);
-                const uint32_t q = (uint32_t)t;
-                if (e < 4) lo |= q << (8 * e); else hi |= q << (8 * (e - 4));
+                const uint32_t q = have ? (uint32_t)t : 0u;
+                c[e / 4] |= q << (8 * (e % 4));
             }
+            unsigned char* cp = sbp + kSbHeader + (size_t)lt * EPL;
+            if (EPL == 16) { u32x4 cv = {c[0], c[1], c[2 % (EPL / 4)], c[3 % (EPL / 4)]}; st_bounce<true>((u32x4*)cp, cv); }
+            else { uint2 cv = {c[0], c[1]}; *(uint2*)cp = cv; }
         }
-        if (EPV == 8) { uint2 c = {lo, hi}; *(uint2*)(sbp + kSbHeader + (size_t)tid * 8) = c; }
-        else *(uint32_t*)(sbp + kSbHeader + (size_t)tid * 4) = lo;
     }
     if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
 }
 
+// What one lane needs of one superblock image to decode its vector: the group's header and its code bytes.
+struct LaneCodes { f32x2 hdr; uint32_t lo, hi; };
 
-__device__ __forceinline__ void decode1(const unsigned char* sbp, unsigned tid, unsigned lpg, int epv, float* r)
+template <int EPV>
+__device__ __forceinline__ LaneCodes load_codes(const unsigned char* sbp, unsigned tid, unsigned lpg)
 {
-    const f32x2 hdr = *(const f32x2*)(sbp + (tid / lpg) * 8);
-    uint32_t lo, hi = 0;
-    if (epv == 8) { const uint2 c = *(const uint2*)(sbp + kSbHeader + (size_t)tid * 8); lo = c.x; hi = c.y; }
-    else lo = *(const uint32_t*)(sbp + kSbHeader + (size_t)tid * 4);
-    for (int e = 0; e < epv; e++) {
-        const uint32_t q = ((e < 4 ? lo >> (8 * e) : hi >> (8 * (e - 4))) & 0xffu);
-        r[e] = __builtin_fmaf((float)q, hdr.x, hdr.y);
+    LaneCodes c;
+    c.hdr = *(const f32x2*)(sbp + (tid / lpg) * 8);
+    c.hi = 0;
+    if (EPV == 8) { const uint2 v = *(const uint2*)(sbp + kSbHeader + (size_t)tid * 8); c.lo = v.x; c.hi = v.y; }
+    else c.lo = *(const uint32_t*)(sbp + kSbHeader + (size_t)tid * 4);
+    return c;
+}
+
+template <int EPV>
+__device__ __forceinline__ void decode_codes(const LaneCodes& c, float* r)
+{
+#pragma unroll
+    for (int e = 0; e < EPV; e++) {
+        const uint32_t q = ((e < 4 ? c.lo >> (8 * e) : c.hi >> (8 * (e - 4))) & 0xffu);
+        r[e] = __builtin_fmaf((float)q, c.hdr.x, c.hdr.y);
     }
 }
 
 // out = T(decode(own image) + decode(received image)); g.a = own image, g.b = received image.  One output vector per
 // lane, so every load and store of a wave is one contiguous run (a lane that owns two consecutive vectors would
-// store with a 32-byte stride, which costs this kernel a quarter of its rate); one superblock per block and iteration.
-template <int DT>
+// store with a 32-byte stride, which costs this kernel a quarter of its rate).  A block takes U superblocks per
+// iteration and issues all their loads before the first store (measured: no gain, see the grid cap's comment).
+template <int DT, int U>
 __global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
 {
     constexpr int EPV = Vec<DT>::EPV;
@@ -233,15 +203,28 @@ __global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
     const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
     const unsigned char* ia = (const unsigned char*)g.a;
     const unsigned char* ib = (const unsigned char*)g.b;
-    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) {
-        const size_t i = sb * blockDim.x + tid;
-        if (i >= nvec) continue;
-        float x[EPV], y[EPV];
-        decode1(ia + sb * kCodecSuperBytes, tid, LPG, EPV, x);
-        decode1(ib + sb * kCodecSuperBytes, tid, LPG, EPV, y);
+    for (size_t sb0 = (size_t)blockIdx.x * U; sb0 < nsb; sb0 += (size_t)gridDim.x * U) {
+        LaneCodes ca[U], cb[U];
+        bool have[U];
 #pragma unroll
-        for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
-        __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + i);
+        for (int u = 0; u < U; u++) {
+            const size_t sb = sb0 + u, i = sb * blockDim.x + tid;
+            have[u] = sb < nsb && i < nvec;
+            if (have[u]) {
+                ca[u] = load_codes<EPV>(ia + sb * kCodecSuperBytes, tid, LPG);
+                cb[u] = load_codes<EPV>(ib + sb * kCodecSuperBytes, tid, LPG);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (!have[u]) continue;
+            float x[EPV], y[EPV];
+            decode_codes<EPV>(ca[u], x);
+            decode_codes<EPV>(cb[u], y);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
+            __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + (sb0 + u) * blockDim.x + tid);
+        }
     }
     if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
@@ -256,9 +239,10 @@ hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const
     return hipGetLastError();
 }
 
-int g_codec_grid_cap = 2048;
+// Measured with 16 MiB bf16, cache-cold (quantise / dequantising sum, us): 2048 blocks 7.3 / 8.1, 1024 blocks 7.1 / 7.9,
+// 512 blocks 8.4 / 9.4; two or four passes' loads issued together (U = 2, 4): 7.5 / 8.4 and 7.9 / 9.0, so U stays 1.
+int g_codec_grid_cap = 1024;
 
-int g_codec_form = 0;           // quantising kernel: 0 = two vectors per lane, 1 = one vector per lane
 
 // spb = superblocks one block takes per iteration
 int codec_grid(size_t nbytes, int dtype, bool gated, size_t spb)
@@ -271,7 +255,7 @@ int codec_grid(size_t nbytes, int dtype, bool gated, size_t spb)
 
 }  // namespace
 
-void set_codec_grid_cap(int cap, int form) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 2048; g_codec_form = form == 1 ? 1 : 0; }
+void set_codec_grid_cap(int cap) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 1024; }
 
 size_t codec_image_bytes(size_t nbytes, int dtype)
 {
@@ -288,19 +272,11 @@ hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timi
     s.bounce = (u32x4*)a.dst; s.cflag = a.cflag; s.pack_arrive = a.arrive;
     s.a = (const u32x4*)a.src; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp; s.sigmode = a.sigmode;
     s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
-    if (g_codec_form == 1) {
-        const int grid1 = codec_grid(a.nbytes, dtype, false, 1);
-        switch (dtype) {
-            case 0: return launch1(k_quant1<0>, grid1, 512, st, t, s);
-            case 1: return launch1(k_quant1<1>, grid1, 256, st, t, s);
-            default: return launch1(k_quant1<2>, grid1, 256, st, t, s);
-        }
-    }
     const int grid = codec_grid(a.nbytes, dtype, false, dtype == 0 ? 1 : 2);
     switch (dtype) {
-        case 0: return launch1(k_quant<0>, grid, (int)kCodecBlock, st, t, s);
-        case 1: return launch1(k_quant<1>, grid, (int)kCodecBlock, st, t, s);
-        default: return launch1(k_quant<2>, grid, (int)kCodecBlock, st, t, s);
+        case 0: return launch1(k_quant<0, 1>, grid, (int)kCodecBlock, st, t, s);
+        case 1: return launch1(k_quant<1, 1>, grid, (int)kCodecBlock, st, t, s);
+        default: return launch1(k_quant<2, 1>, grid, (int)kCodecBlock, st, t, s);
     }
 }
 
@@ -317,9 +293,9 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
     s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
     const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr, 1);
     switch (q.dtype) {
-        case 0: return launch1(k_sum_quant<0>, grid, 512, st, t, s);
-        case 1: return launch1(k_sum_quant<1>, grid, 256, st, t, s);
-        default: return launch1(k_sum_quant<2>, grid, 256, st, t, s);
+        case 0: return launch1(k_sum_quant<0, 1>, grid, 512, st, t, s);
+        case 1: return launch1(k_sum_quant<1, 1>, grid, 256, st, t, s);
+        default: return launch1(k_sum_quant<2, 1>, grid, 256, st, t, s);
     }
 }
 

@@ -21,6 +21,7 @@
 #include <algorithm>
 
 #include "tbv_dma.h"
+#include "tbv_sock.h"
 
 namespace tbv {
 
@@ -146,7 +147,7 @@ void* progress_rail(void* arg)
         if (posted < tail) { posted = tail; t_watch = 0; }
 
         const Item& oldest = x.q[tail % NS];
-        const bool one_at_a_time = G.hooks || !G.gpusig || oldest.host_wire || G.err.load(std::memory_order_relaxed);
+        const bool one_at_a_time = G.hooks || !G.gpusig || oldest.host_wire || G.peer_tcp || G.err.load(std::memory_order_relaxed);
         if (one_at_a_time && posted == tail) {
             const Item it = oldest;
             if (G.gpusig) {
@@ -168,7 +169,7 @@ void* progress_rail(void* arg)
         // several postings (a posting is a kernel launch, 3 us and more)
         if (posted < head && !G.err.load(std::memory_order_relaxed)) {
             const Item& it = x.q[posted % NS];
-            if (!it.host_wire && !G.hooks) {                         // else it goes one at a time, once it is the oldest
+            if (!it.host_wire && !G.hooks && !G.peer_tcp) {          // else it goes one at a time, once it is the oldest
                 if (t_watch == 0) t_watch = nowt();
                 if (pack_complete(x, it, t_watch, NS) == 1) {
                     const int k = (int)(posted % NS);
@@ -352,9 +353,10 @@ int configure(const char* devs, size_t cap)
     // a call whose peer payload has not arrived yet, above the one-kernel size: pack blocks + gated sum blocks in one launch
     G.staged_merge = geti("TBV_STAGEDMERGE", 1);
     G.force_gate = geti("TBV_FORCEGATE", 0);
+    { const char* e = getenv("TBV_PEER"); G.peer_tcp = (e && !strcmp(e, "tcp")) ? 1 : 0; }
     set_gated_tuning(geti("TBV_GATEDGRID", 0), geti("TBV_GATEDUNROLL", 0));
     set_row_grid_cap(geti("TBV_ROWGRID", 0));
-    set_codec_grid_cap(geti("TBV_CODECGRID", 0), geti("TBV_CODECFORM", 0));
+    set_codec_grid_cap(geti("TBV_CODECGRID", 0));
     G.codec = geti("TBV_CODEC", 0);
     G.codec_min = getz("TBV_CODEC_MIN", (size_t)512 << 10);
     // Cache-hint profile: when both rings plus one local and one output tensor fit in three quarters of the
@@ -647,9 +649,10 @@ int drain_rails()
 
 // ---- initialisation and teardown (allocation half of tbv_ar_init, step4/libtbvcoll.cpp:279-342,405-413) ----
 
-int init_impl(int rank, const char* devs, size_t cap)
+int init_impl(int rank, const char* devs, const char* peer_ip, int port, size_t cap)
 {
     if (configure(devs, cap) != 0) return -1;
+    if (G.peer_tcp && rank != 0 && rank != 1) FAIL("two-process mode has ranks 0 and 1, not %d", rank);
     G.rank = rank;
     if (hipGetDevice(&G.device) != hipSuccess) FAIL("no HIP device");
     { int v = 0;
@@ -695,6 +698,9 @@ int init_impl(int rank, const char* devs, size_t cap)
         G.can_write_value = 0;
     }
     G.seq = 0; G.err.store(0);
+    // two processes on this GPU: meet the peer before any thread of this rank starts (as the reference brings its
+    // queue pairs up before it spawns its progress threads, step4/libtbvcoll.cpp:371-407)
+    if (G.peer_tcp && sock_start(rank, peer_ip, port) != 0) return -1;
     if (G.async) {
         G.run.store(1);
         for (int r = 0; r < G.R; r++) {
@@ -705,8 +711,8 @@ int init_impl(int rank, const char* devs, size_t cap)
     G.inited = 1;
     LOGF("rank%d ready: %d rail(s), cap=%zu KiB, %d slots, mode %s", rank, G.R, G.cap / 1024, G.nslot,
          G.async ? (G.gpusig ? (G.kwait ? "ASYNC+GPUSIG+KWAIT" : "ASYNC+GPUSIG") : "ASYNC+EVENT") : "SYNC");
-    LOGF("  emulated peer on device %d; stream wait value %s, stream write value %s; uncached=%d tag=%d railsum=%d fuse=%d fusewait<=%zu",
-         G.device, G.can_wait_value ? "yes" : "no (wait kernel)", G.can_write_value ? "yes" : "no (mark kernel)",
+    LOGF("  %s on device %d; stream wait value %s, stream write value %s; uncached=%d tag=%d railsum=%d fuse=%d fusewait<=%zu",
+         G.peer_tcp ? "peer = a second process" : "emulated peer", G.device, G.can_wait_value ? "yes" : "no (wait kernel)", G.can_write_value ? "yes" : "no (mark kernel)",
          G.uncached, G.tag, G.railsum, G.fuse, G.fusewait_max);
     LOGF("  wire %s; copy-engine access for the host wire: %s", G.wire_mode == 1 ? "stream" : G.wire_mode == 2 ? "host" : "auto", dma ? "yes" : "no");
     LOGF("  small calls (<= %zu B) in one kernel: %s", G.fusewait_max, G.onekernel ? "yes" : "no");
@@ -735,6 +741,7 @@ void teardown()
     // let the GPU finish what is queued (flags are raised even after an error), then stop the threads
     (void)hipDeviceSynchronize();
     stop_progress();
+    sock_stop();
     for (int r = 0; r < MAXRAIL; r++) if (G.rr[r].wire) { (void)hipStreamDestroy(G.rr[r].wire); G.rr[r].wire = nullptr; }
     peer_teardown();
     if (G.util) { (void)hipStreamDestroy(G.util); G.util = nullptr; }

@@ -80,6 +80,7 @@ struct Engine {
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     int merge = 1;                            // resident peer: pack and sum blocks in one launch (TBV_MERGE)
     size_t merge_max = (size_t)256 << 20;     // TBV_MERGEMAX: largest payload that takes the merged launch
+    int peer_tcp = 0;                         // TBV_PEER=tcp: the peer is a second process on this GPU, reached over TCP (tbv_sock.cpp)
     int force_gate = 0;                       // measurement aid: early-peer large calls take the gated one-launch form (TBV_FORCEGATE)
     int staged_merge = 1;                     // peer not there yet: pack blocks + gated sum blocks in one launch (TBV_STAGEDMERGE)
     int streaming = 0;                        // cache-hint profile of the large kernels (TBV_STREAMING, default by ring size)
@@ -202,7 +203,7 @@ inline int rails_for(size_t nbytes) { return nbytes <= G.rail1max ? 1 : G.R; }
 
 // ---- tbv_engine.cpp -------------------------------------------------------------------
 int configure(const char* devs, size_t cap);
-int init_impl(int rank, const char* devs, size_t cap);
+int init_impl(int rank, const char* devs, const char* peer_ip, int port, size_t cap);
 void teardown();
 void stop_progress();
 int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipStream_t st, Call* c, const NormArgs* nm = nullptr,

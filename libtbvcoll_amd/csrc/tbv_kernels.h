@@ -113,7 +113,7 @@ static constexpr unsigned kCodecGroup = 128;
 static constexpr unsigned kCodecSuper = 2048;          // elements per superblock
 static constexpr unsigned kCodecSuperBytes = 2176;     // 16 x 8 header bytes + 2048 code bytes
 size_t codec_image_bytes(size_t nbytes, int dtype);
-void set_codec_grid_cap(int cap, int form);            // most blocks of a codec launch (0 = default); form of the quantising kernel
+void set_codec_grid_cap(int cap);                      // most blocks of a codec launch (0 = default)
 hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum_quant(const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
 

@@ -18,6 +18,7 @@
 
 #include "../../include/tbvcoll_emu.h"
 #include "tbv_dma.h"
+#include "tbv_sock.h"
 
 namespace tbv {
 
@@ -49,7 +50,7 @@ int host_deposit(Rail& x, const Item& it, size_t off, size_t len, double t0)
     const size_t ck = G.chunkb ? G.chunkb : (n ? n : 1);
     int rc = 0;
     for (size_t o = 0; o < n && rc == 0; o += ck)
-        rc = dma_copy(x.idx, slot_recv(it.slot) + off + o, DMA_DEVICE, src + o, DMA_DEVICE, std::min(ck, n - o), left());
+        rc = dma_copy(x.idx, slot_recv(it.slot) + off + o, DMA_DEVICE, src + o, G.peer_tcp ? DMA_HOST : DMA_DEVICE, std::min(ck, n - o), left());
     if (rc == 0 && it.peer && G.tag) {       // the peer's own tag travels at the end of its payload
         const size_t to = tag_offset(it.nbytes);
         if (to >= off && to < off + len)
@@ -258,15 +259,25 @@ int wire_xfer(Rail& x, const Item& it)
         }
     }
 
-    if (!it.resident && it.host_wire) {
+    // Two processes: this rail's fragment goes to the peer over its connection and the peer's comes back into pinned
+    // host memory; from there it is deposited like an emulated peer's payload (same copy, same arrival word).
+    Item tcp_item = it;
+    if (G.peer_tcp) {
+        const char* staged = nullptr;
+        if (sock_exchange(x, it, off, len, t0, &staged) != 0) return -1;
+        tcp_item.peer = staged - off;               // the deposit adds the fragment's offset
+        tcp_item.resident = false;
+    }
+    const Item& dep = G.peer_tcp ? tcp_item : it;
+    if (!dep.resident && dep.host_wire) {
         // Host wire: the fragment goes straight into the receive slot with a copy-engine transfer that
         // this thread waits for, and this thread raises the arrival word itself.  Nothing is placed on
         // one of our compute queues, so this works even when the caller's gated stream and the side
         // stream are multiplexed onto the same hardware queue.
-        if (host_deposit(x, it, off, len, t0) != 0) return -1;
+        if (host_deposit(x, dep, off, len, t0) != 0) return -1;
         if (!withheld) st_rel(aw, it.seq);
-    } else if (!it.resident) {
-        if (stream_deposit(x, it, off, len, withheld) != 0) return -1;
+    } else if (!dep.resident) {
+        if (stream_deposit(x, dep, off, len, withheld) != 0) return -1;
     } else if (!withheld) {
         st_rel(aw, it.seq);                  // payload already in place: arrival is immediate
     }
@@ -280,6 +291,7 @@ int wire_xfer(Rail& x, const Item& it)
             return -1;
         }
     }
+    if (G.peer_tcp) sock_consumed(x, it);
     account_arrival(x, it, t0, tp, nowt());      // logged before the next rail in the script may go
     if (my_turn != (size_t)-1) G.turn.store(my_turn + 1, std::memory_order_release);
     return 0;
@@ -323,6 +335,7 @@ int peer_assign(Call* c, size_t nbytes, int dtype, const char** peer)
 {
     *peer = nullptr;
     c->resident = false;
+    if (G.peer_tcp) return 0;                    // the payload comes from the peer process, over the wire
     bool from_resident = false;
     if (!G.staged.empty()) {
         Staged s = G.staged.front(); G.staged.pop_front();
@@ -377,6 +390,7 @@ using namespace tbv;
 extern "C" int tbv_emu_stage_peer(const void* src, size_t nbytes)
 {
     if (!G.inited || !src) return -1;
+    if (G.peer_tcp) FAIL("two-process mode: the peer's payload comes from the peer process, it cannot be staged");
     if (G.staged.size() >= LOG_MAX) return -1;
     reap_owned();
     const bool host = pointer_is_host(src);
@@ -389,6 +403,7 @@ extern "C" int tbv_emu_stage_peer(const void* src, size_t nbytes)
 extern "C" int tbv_emu_stage_peer_repeat(const void* src, size_t nbytes)
 {
     if (!G.inited) return -1;
+    if (G.peer_tcp && src) FAIL("two-process mode: the peer's payload comes from the peer process, it cannot be staged");
     if (src && pointer_is_host(src)) { src = to_device(src, nbytes); if (!src) return -1; G.owned.back().second = ~0ull; }   // kept until shutdown
     G.repeat = Staged{(const char*)src, src ? nbytes : 0, false};
     return 0;
@@ -401,6 +416,7 @@ extern "C" int tbv_emu_stage_peer_repeat(const void* src, size_t nbytes)
 extern "C" int tbv_emu_peer_resident(const void* src, size_t nbytes)
 {
     if (!G.inited) return -1;
+    if (G.peer_tcp && src) FAIL("two-process mode: the peer's payload comes from the peer process, it cannot be made resident");
     if (src && nbytes > G.cap) return -2;
     if (drain_rails() != 0) return -1;
     if (hipDeviceSynchronize() != hipSuccess) return -1;        // no earlier sum may still be reading a slot or the old copy

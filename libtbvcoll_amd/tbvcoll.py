@@ -46,6 +46,7 @@ _SIGNATURES = {
     "tbv_emu_stage_peer": (_I, [_VP, _SZ]), "tbv_emu_stage_peer_repeat": (_I, [_VP, _SZ]), "tbv_emu_peer_resident": (_I, [_VP, _SZ]),
     "tbv_emu_arrival_script": (_I, [_PI, _SZ]), "tbv_emu_withhold": (_I, [_U64, _I]), "tbv_emu_hold_rail": (_I, [_I, _I]),
     "tbv_emu_seq": (_U64, []), "tbv_emu_plan": (_I, [_SZ, _PSZ, _PSZ]), "tbv_emu_configure": (_I, [ctypes.c_char_p, _SZ]),
+    "tbv_emu_rendezvous": (_I, [_I, ctypes.c_char_p, _I, ctypes.c_double]),
     "tbv_emu_nslot": (_I, []), "tbv_emu_stride": (_SZ, []), "tbv_emu_send_slot": (_VP, [_I]), "tbv_emu_recv_slot": (_VP, [_I]),
     "tbv_emu_arrival_log": (_SZ, [_PU, _PI, _SZ]),
     "tbv_emu_latency_probe": (_I, [_I]), "tbv_emu_latencies": (_SZ, [_PD, _SZ]),
