@@ -91,6 +91,9 @@ size_t tbv_emu_latencies(double* us, size_t max);
  * launches and their mean and minimum duration in microseconds, then forgets them. */
 int tbv_emu_kernel_timing(int on);
 size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_us);
+/* The recorded launches one by one: start and end of each, in microseconds after the start of the first
+ * (up to `max`; the samples are kept).  Shows where a short burst of calls loses time between launches. */
+size_t tbv_emu_kernel_timeline(int which, double* start_us, double* stop_us, size_t max);
 
 /* GPU footprints (kept with TBV_KWAIT=1, as the reference's, step4/libtbvcoll.cpp:98):
  * sequence numbers of the last [wait entered, wait passed, pack started, sum done,

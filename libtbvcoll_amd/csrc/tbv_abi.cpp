@@ -214,6 +214,22 @@ extern "C" size_t tbv_emu_kernel_times(int which, double* mean_us, double* min_u
     return n;
 }
 
+// Start and end of every recorded launch of one kind, in microseconds after the start of the first one (the
+// dispatches' own timestamps); synchronises the device and keeps the samples.  Returns how many were written.
+extern "C" size_t tbv_emu_kernel_timeline(int which, double* start_us, double* stop_us, size_t max)
+{
+    if (!G.inited || which < 0 || which > 1 || !start_us || !stop_us) return 0;
+    (void)hipDeviceSynchronize();
+    size_t n = 0;
+    for (size_t i = 0; i < G.kev_used[which] && n < max; i++) {
+        float a = 0, b = 0;
+        if (hipEventElapsedTime(&a, G.kev[which][0].first, G.kev[which][i].first) != hipSuccess ||
+            hipEventElapsedTime(&b, G.kev[which][0].first, G.kev[which][i].second) != hipSuccess) continue;
+        start_us[n] = a * 1e3; stop_us[n] = b * 1e3; n++;
+    }
+    return n;
+}
+
 extern "C" void tbv_emu_footprints(unsigned long long out[5])
 {
     for (int i = 0; i < 5; i++) out[i] = G.inited ? footprints()[i] : 0;

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "tbv_emu_arrival_log": (_SZ, [_PU, _PI, _SZ]),
     "tbv_emu_latency_probe": (_I, [_I]), "tbv_emu_latencies": (_SZ, [_PD, _SZ]),
     "tbv_emu_kernel_timing": (_I, [_I]), "tbv_emu_kernel_times": (_SZ, [_I, _PD, _PD]),
+    "tbv_emu_kernel_timeline": (_SZ, [_I, _PD, _PD, _SZ]),
     "tbv_emu_footprints": (None, [_PU]), "tbv_emu_tag_counts": (None, [_PU, _PU, _PU]),
     "tbv_ar_allreduce_chunked": (_I, [_VP, _VP, _SZ, _I, _VP]),
     "tbv_emu_run_pack": (_I, [_VP, _SZ, _I, _VP]), "tbv_emu_run_sum": (_I, [_VP, _VP, _VP, _SZ, _I, _VP]),
@@ -262,6 +263,13 @@ def kernel_times(which):
     m, mn = ctypes.c_double(), ctypes.c_double()
     n = _lib.tbv_emu_kernel_times(which, ctypes.byref(m), ctypes.byref(mn))
     return n, m.value, mn.value
+
+
+def kernel_timeline(which, max_n=4096):
+    """[(start_us, stop_us)] of the recorded launches, relative to the start of the first; keeps the samples."""
+    a, b = (ctypes.c_double * max_n)(), (ctypes.c_double * max_n)()
+    n = _lib.tbv_emu_kernel_timeline(which, a, b, max_n)
+    return [(a[i], b[i]) for i in range(n)]
 
 
 def hbm_probe(kind, nbytes, pool_bytes, reps, so=_DEFAULT_SO):
