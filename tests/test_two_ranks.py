@@ -124,7 +124,8 @@ def run_two_ranks(env_common, timeout=240):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("env", [{}, {"TBV_ASYNC": 0}, {"TBV_STAGEDMERGE": 0, "TBV_ONEKERNEL": 0, "TBV_FUSEWAIT": 0}])
+@pytest.mark.parametrize("env", [{}, {"TBV_ASYNC": 0}, {"TBV_STAGEDMERGE": 0, "TBV_ONEKERNEL": 0, "TBV_FUSEWAIT": 0}, {"TBV_TAG": 1},
+                                 {"TBV_RAILSUM": 1}, {"TBV_WIRE": "host"}, {"TBV_CHUNK": 65536, "TBV_UNCACHED": 1}, {"DEVS": "a,b,c"}])
 def test_two_processes_exact(env):
     """The counterpart of step4/test_exact.py as two processes on the one GPU: 9 dtype x size cells, both references."""
     from gpu_util import say
