@@ -255,6 +255,7 @@ struct StepArgs {
     unsigned long long* pack_relay;   // device word: the pack part stores seq here when its last block is done; the sum part of
                                       // the same launch waits for it (beside its flag) when the output aliases the local tensor
     int b_uncached;             // the received payload lies in uncached memory: the gate needs no cache invalidation
+    unsigned tiles;             // sum part of a pipeline launch: tiles of blockDim x US vectors, taken in turn by its blocks
 };
 
 }  // namespace tbv

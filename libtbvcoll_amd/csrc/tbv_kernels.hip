@@ -23,6 +23,27 @@ namespace tbv {
 // 1 KiB of consecutive memory and a lane has U (x2 for the sum) loads in flight.
 
 
+// The bytes past the last whole vector (at most 15), by the first lanes of one block.
+template <int DT, bool PACK, bool SUM>
+__device__ __forceinline__ void step_tail(const StepArgs& g)
+{
+    const unsigned tid = threadIdx.x;
+    const unsigned tail = (unsigned)(g.nbytes & 15);
+    if (!tail) return;
+    const size_t off = (g.nbytes >> 4) << 4;
+    if (PACK && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
+    if (SUM) {
+        typedef typename Elem<DT>::T T;
+        const unsigned ne = tail / sizeof(T);
+        if (tid < ne) {
+            const T* pa = (const T*)((const char*)g.a + off);
+            const T* pb = (const T*)((const char*)g.b + off);
+            T* po = (T*)((char*)g.out + off);
+            po[tid] = Elem<DT>::add(pa[tid], pb[tid]);
+        }
+    }
+}
+
 // Block `bid` of `nblk` does its share of the payload; block 0 also does the bytes past the last whole vector.
 template <int DT, int U, bool PACK, bool SUM, bool STREAM>
 __device__ __forceinline__ void step_body(const StepArgs& g, unsigned bid, unsigned nblk)
@@ -58,21 +79,7 @@ __device__ __forceinline__ void step_body(const StepArgs& g, unsigned bid, unsig
             }
         }
     }
-    const unsigned tail = (unsigned)(g.nbytes & 15);
-    if (tail && bid == 0) {
-        const size_t off = nvec << 4;
-        if (PACK && tid < tail) ((unsigned char*)g.bounce)[off + tid] = ((const unsigned char*)g.a)[off + tid];
-        if (SUM) {
-            typedef typename Elem<DT>::T T;
-            const unsigned ne = tail / sizeof(T);
-            if (tid < ne) {
-                const T* pa = (const T*)((const char*)g.a + off);
-                const T* pb = (const T*)((const char*)g.b + off);
-                T* po = (T*)((char*)g.out + off);
-                po[tid] = Elem<DT>::add(pa[tid], pb[tid]);
-            }
-        }
-    }
+    if (bid == 0) step_tail<DT, PACK, SUM>(g);
 }
 
 template <int DT, int U, bool PACK, bool SUM, bool STREAM>
@@ -152,9 +159,13 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_pipe(StepArgs pk, StepArgs
             if (last && pk.pack_relay) __hip_atomic_store(pk.pack_relay, pk.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         }
     } else {
-        const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
+        // The sum part works on `tiles` tiles of blockDim x US vectors; its blocks (capped in number, because a waiting
+        // block holds its wave slots) take tiles bid, bid + S, ...  (Tried and dropped, neither changed the 14.0 us of a
+        // 16 MiB launch whose flag is up beforehand: blocks behind the waiting ones that look at the relay once and take
+        // the waiting blocks' second tiles if it is up; loading the first tile of the local tensor ahead of the gate.)
+        const unsigned bid = blockIdx.x - P, S = gridDim.x - P, T = sm.tiles;
         if (sm.wait_flag) gate_wait_as(bid, sm.wait_flag, sm.seq, sm.spin_limit, sm.relay, sm.fp, !sm.b_uncached, sm.pack_relay, true);
-        step_body<DT, US, false, true, STREAM>(sm, bid, S);     // few blocks wait: each keeps several loads per operand in flight
+        for (unsigned t = bid; t < T; t += S) step_body<DT, US, false, true, STREAM>(sm, t, T);
         if (sm.done) grid_complete(sm.done, sm.seq, sm.done_arrive, bid, S, 1);
     }
 }
@@ -271,6 +282,16 @@ static bool g_grid_cap_given = false;   // a cap from the environment applies to
 static int g_block = kThreads;
 static bool g_stream = false;   // streaming profile (see the cache hints above)
 static int g_gated_cap = kGatedMaxGrid;     // most blocks of a grid (or part of one) that waits for a flag inside
+// The cap is held in waves as well: whatever block size is in use, the waiting part of a grid never takes more than half
+// of the GPU's 8192 wave slots (a cap counted in blocks alone would let 1024 blocks of 512 lanes fill every slot, and the
+// kernel whose completion raises the flag could then never be placed).
+static constexpr int kGatedMaxWaves = 4096;
+static inline int gated_cap_for(int block)
+{
+    const int by_waves = kGatedMaxWaves / ((block + 63) / 64);
+    const int cap = g_gated_cap < by_waves ? g_gated_cap : by_waves;
+    return cap < 1 ? 1 : cap;
+}
 static int g_gated_unroll = 2;
 
 struct Geom { int grid, block, unroll; };
@@ -401,12 +422,12 @@ hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t)
         s.a = (const u32x4*)a.a; s.nbytes = a.nbytes; s.seq = a.seq; s.fp = a.fp;
         s.pre_word = a.pre.word; s.pre_seq = a.pre.seq;
         Geom g = geom_for(a.nbytes);
-        if (a.wait_flag && g.grid > g_gated_cap) g.grid = g_gated_cap;
+        if (a.wait_flag && g.grid > gated_cap_for(g.block)) g.grid = gated_cap_for(g.block);
         return launch_step<false, true>(a.dtype, s, g, st, t);
     }
     size_t esz = a.dtype == 0 ? 4 : 2, n = a.nbytes / esz;
     int grid = (int)((n + kThreads - 1) / kThreads); if (grid > kMaxGrid) grid = kMaxGrid; if (grid < 1) grid = 1;
-    if (a.wait_flag && grid > g_gated_cap) grid = g_gated_cap;
+    if (a.wait_flag && grid > gated_cap_for(kThreads)) grid = gated_cap_for(kThreads);
     switch (a.dtype) {
         case 0: return launch1(k_sum_narrow<0>, grid, kThreads, st, t, a);
         case 1: return launch1(k_sum_narrow<1>, grid, kThreads, st, t, a);
@@ -524,12 +545,17 @@ hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, cons
     const size_t pvec = p.nbytes >> 4, svec = q.nbytes >> 4;
     const int up = pvec >= (size_t)2 * block * 1024 ? 2 : 1;
     const int us = q.wait_flag ? g_gated_unroll : 4;
-    int P = (int)((pvec + (size_t)block * up - 1) / ((size_t)block * up)), S = (int)((svec + (size_t)block * us - 1) / ((size_t)block * us));
+    int P = (int)((pvec + (size_t)block * up - 1) / ((size_t)block * up));
     if (P < 1) P = 1;
-    if (S < 1) S = 1;
     const int pcap = g_grid_cap_given ? g_grid_cap : 2048;
     if (P > pcap) P = pcap;
-    if (S > (q.wait_flag ? g_gated_cap : g_grid_cap)) S = q.wait_flag ? g_gated_cap : g_grid_cap;
+    // sum part: T tiles, taken in turn by at most `wcap` blocks (see k_pipe)
+    size_t T = (svec + (size_t)block * us - 1) / ((size_t)block * us);
+    if (T < 1) T = 1;
+    if (T > 0x7fffffffu) return hipErrorInvalidValue;
+    const size_t wcap = (size_t)(q.wait_flag ? gated_cap_for(block) : g_grid_cap);
+    const int S = (int)(T < wcap ? T : wcap);
+    sm.tiles = (unsigned)T;
     pk.pack_blocks = (unsigned)P;
     if (g_stream) {
         switch (q.dtype) {

@@ -286,7 +286,7 @@ inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 // Most blocks of a row-kernel launch: 0 = what is resident at once (see launch_row_norm), else a given number.
 // Every block counted by grid_complete needs a place in the counter lines, which hold 8128 blocks.
 int g_row_grid_cap = 0;
-constexpr int kRowGatedCap = 512;       // a grid that waits for its flag inside: 512 x 4 waves, a quarter of the GPU's wave slots
+constexpr int kRowGatedWaves = 2048;    // a grid that waits for its flag inside holds at most a quarter of the GPU's 8192 wave slots
 
 }  // namespace
 
@@ -331,7 +331,8 @@ hipError_t launch_row_norm(int mode, const PackArgs* p, const SumArgs& q, const 
     // construction (its row count is bounded).
     // (the norm-only form needs fewer registers: all 8192 wave slots hold a block of it)
     int cap = g_row_grid_cap > 0 ? g_row_grid_cap : (mode == 0 ? 8192 : 4096) / (block / 64);
-    if (mode == 1 && q.wait_flag && cap > kRowGatedCap) cap = kRowGatedCap;
+    const int gated_cap = kRowGatedWaves / (block / 64);
+    if (mode == 1 && q.wait_flag && cap > gated_cap) cap = gated_cap;
     if (cap < 1) cap = 1;
     const unsigned per_block = (nm.rows + (unsigned)cap - 1) / (unsigned)cap;
     const int grid = mode == 2 ? (int)nm.rows : (int)((nm.rows + per_block - 1) / per_block);

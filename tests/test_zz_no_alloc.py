@@ -104,6 +104,47 @@ def test_no_alloc_step_without_init():
         assert int(words[0]) == seq and int(words[8]) == seq
 
 
+FIRST_CALL_UNDER_CAPTURE = r"""
+import ctypes, sys
+sys.path.insert(0, {root!r})
+import torch
+from libtbvcoll_amd import tbvcoll
+lib = tbvcoll.load()                       # no tbv_ar_init, no earlier step: the counters' address is not bound yet
+n = 1 << 20
+a = torch.ones(n // 2, dtype=torch.bfloat16, device="cuda"); b = torch.full_like(a, 2.0)
+out = torch.zeros_like(a); bounce = torch.zeros_like(a)
+side = torch.cuda.Stream()
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g, stream=side):
+    out.zero_()                            # something of the program's own, so the graph is not empty
+    rc = lib.tbv_step_noalloc(out.data_ptr(), a.data_ptr(), b.data_ptr(), bounce.data_ptr(), 0, n, 2, None, None, 1,
+                              torch.cuda.current_stream().cuda_stream)
+print("CAPTURED_RC", rc, flush=True)
+g.replay(); torch.cuda.synchronize()
+print("AFTER_REPLAY", float(out.float().abs().max()), flush=True)
+rc = lib.tbv_step_noalloc(out.data_ptr(), a.data_ptr(), b.data_ptr(), bounce.data_ptr(), 0, n, 2, None, None, 2,
+                          torch.cuda.current_stream().cuda_stream)
+torch.cuda.synchronize()
+print("EAGER_RC", rc, bool(torch.equal(out, a + b)), flush=True)
+"""
+
+
+def test_first_no_alloc_step_inside_a_capture_is_refused():
+    """The first call on a device looks up the address of the built-in counters, which is not allowed while a stream is
+    being captured: such a call is refused with -1 (and launches nothing) instead of breaking the capture.  Needs a
+    process in which neither tbv_ar_init nor an earlier step has run, hence the child process."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    say("first no-alloc step under capture, in a fresh process")
+    p = subprocess.run([sys.executable, "-c", FIRST_CALL_UNDER_CAPTURE.format(root=root)], capture_output=True, text=True, timeout=240)
+    assert "CAPTURED_RC -1" in p.stdout, (p.stdout, p.stderr[-2000:])
+    assert "inside a stream capture" in p.stderr
+    assert "AFTER_REPLAY 0.0" in p.stdout                        # the refused call recorded nothing into the graph
+    assert "EAGER_RC 0 True" in p.stdout, (p.stdout, p.stderr[-2000:])
+
+
 @pytest.mark.parametrize("uncached", [0, 1])
 def test_no_alloc_step_in_a_graph(uncached):
     """Recorded into a HIP graph (the callers the entry point is for) and replayed four times with the program's own
