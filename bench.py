@@ -157,8 +157,14 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
         timed(min(steps, 48))
     tbv.stats4()                       # drop what the warm-up (and the first call's stream probe) accumulated
     wall = timed(steps)
-    timed(steps, events=True)          # the same region once more, with the two events in it
-    ev_timed_us = ev_us[0]
+    # the same region again with the two events in it; a region of few steps is repeated and the median taken, since one
+    # host hiccup inside a 20-step region moves its average by several percent
+    ev_runs = []
+    for _ in range(5 if steps <= 500 else 1):
+        timed(steps, events=True)
+        if ev_us[0]:
+            ev_runs.append(ev_us[0])
+    ev_timed_us = sorted(ev_runs)[len(ev_runs) // 2] if ev_runs else None
     tbv.stats4()
     # what the region costs beside its steps: a second region of twice the steps gives slope and intercept
     region = None
@@ -207,7 +213,7 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     for k, _ in env:
         os.environ.pop(k, None)
     return {"wall": wall, "steps": steps, "long_wall": long_wall, "long_steps": long_steps, "ok": ok and not err, "enq_us": enq,
-            "ev_us": ev_timed_us, "ev_long_us": ev_long_us, "region": region,
+            "ev_us": ev_timed_us, "ev_runs": ev_runs, "ev_long_us": ev_long_us, "region": region,
             "pack_us": pack_us, "pack_min_us": pack_min, "n_pack": n_pack, "sum_us": sum_us, "sum_min_us": sum_min, "n_sum": n_sum}
 
 
@@ -557,11 +563,12 @@ def main():
         timing = "dispatch timestamps of every sum launch in a further pass of the same steps"
     else:
         roof = kernel_roofline(dom_bytes, cold["ev_us"] or cold["sum_us"], cold["sum_min_us"], max(args.steps - 1, 1), ceiling) or {}
+        roof["avg_launch_us_regions"] = [round(x, 3) for x in cold["ev_runs"]]
         roof["per_dispatch_timestamps"] = {"avg_us": round(cold["sum_us"], 3), "min_us": round(cold["sum_min_us"], 3), "launches": cold["n_sum"],
                                            "frac": round(dom_bytes / (cold["sum_us"] * 1e-6) / HBM_PEAK, 4) if cold["sum_us"] else None}
-        timing = ("avg_launch_us: the timed region run once more right after the host-clocked one, with two events on the caller's stream "
-                  "around the launches after the first, device time / (steps - 1) (the event records cost a region about 10 us, so they "
-                  "stay out of the host-clocked one); per_dispatch_timestamps: start and end stamps of every launch in a further pass "
+        timing = ("avg_launch_us: the timed region run again right after the host-clocked one, with two events on the caller's stream "
+                  "around the launches after the first, device time / (steps - 1); median of the regions listed in avg_launch_us_regions "
+                  "(the event records cost a region about 10 us, so they stay out of the host-clocked one); per_dispatch_timestamps: start and end stamps of every launch in a further pass "
                   "(what a kernel trace averages)")
     roof["denominator"] = ("4N: the local tensor is read once" if fused_headline else "3N (sum kernel alone)" if two_headline else
                            "5N = pack 2N + sum 3N algorithmic bytes; the sum blocks' read of the local tensor is issued but served by the L2, see frac_fabric")

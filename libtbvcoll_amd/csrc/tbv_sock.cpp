@@ -270,9 +270,9 @@ int sock_start(int rank, const char* peer_ip, int port)
     if (sock_rendezvous(rank, peer_ip, port, fds, timeout_s) != 0) return -1;
     S.buf_bytes = G.stride;
     S.err.store(0);
+    for (int r = 0; r < G.R; r++) S.r[r].fd = fds[r];     // owned by sock_stop() from here on, whatever fails below
     for (int r = 0; r < G.R; r++) {
         SockRail& x = S.r[r];
-        x.fd = fds[r];
         if (hipHostMalloc((void**)&x.tx, S.buf_bytes, hipHostMallocDefault) != hipSuccess) FAIL("two-process wire: pinned staging allocation failed");
         for (int s = 0; s < G.nslot; s++) {
             if (hipHostMalloc((void**)&x.rx[s], S.buf_bytes, hipHostMallocDefault) != hipSuccess) FAIL("two-process wire: pinned staging allocation failed");
