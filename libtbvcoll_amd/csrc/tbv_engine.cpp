@@ -350,6 +350,7 @@ int configure(const char* devs, size_t cap)
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
     G.merge = geti("TBV_MERGE", 1);
     G.merge_max = getz("TBV_MERGEMAX", (size_t)256 << 20);
+    set_merge_segment(G.merge_max);
     // a call whose peer payload has not arrived yet, above the one-kernel size: pack blocks + gated sum blocks in one launch
     G.staged_merge = geti("TBV_STAGEDMERGE", 1);
     G.force_gate = geti("TBV_FORCEGATE", 0);
@@ -421,10 +422,9 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                                     (nm ? nm->rows <= (unsigned)kRowNormMaxSmallRows : small_call_blocks(nbytes) <= kSmallCallMaxBlocks);
             // Payload already in place and too large for the one-kernel call: pack blocks and sum blocks in one
             // launch (a launch costs about 2.4 us of stream time whatever it does).
-            // (up to a size: the two halves share the local tensor through the L2 only while they stay close in time;
-            // at 1 GiB the merged launch moves 5.1-5.45 TB/s, two launches 5.6)
-            const bool mergeable = G.merge && !fuse_wanted && !one_kernel && in_place_already && !gate_resident && plain && G.packsig == 0 && !nm &&
-                                   nbytes <= G.merge_max;
+            // (payloads beyond TBV_MERGEMAX as several such launches, one per segment: the two halves share the local
+            // tensor through the L2 only while they stay close in time)
+            const bool mergeable = G.merge && !fuse_wanted && !one_kernel && in_place_already && !gate_resident && plain && G.packsig == 0 && !nm;
             // Pack blocks and sum blocks read the local tensor independently, so a sum block may store out[i] before
             // the pack block has read a[i]: an output that overlaps the local tensor cannot take the merged launch.
             // In place it takes the fused body instead (one lane loads a[i] once and does both stores); any other

@@ -79,7 +79,7 @@ struct Engine {
     int configured = 0, inited = 0, rank = 0, R = 0, async = 1, nslot = 8, gpusig = 1, kwait = 0;
     int uncached = 1, tag = 0, cpu = -1, wr_hwm = 8, device = 0, railsum = 0, fuse = 0, packsig = 0;
     int merge = 1;                            // resident peer: pack and sum blocks in one launch (TBV_MERGE)
-    size_t merge_max = (size_t)256 << 20;     // TBV_MERGEMAX: largest payload that takes the merged launch
+    size_t merge_max = (size_t)256 << 20;     // TBV_MERGEMAX: largest payload of one merged or staged launch (larger early-peer calls: one merged launch per segment)
     int peer_tcp = 0;                         // TBV_PEER=tcp: the peer is a second process on this GPU, reached over TCP (tbv_sock.cpp)
     int force_gate = 0;                       // measurement aid: early-peer large calls take the gated one-launch form (TBV_FORCEGATE)
     int staged_merge = 1;                     // peer not there yet: pack blocks + gated sum blocks in one launch (TBV_STAGEDMERGE)

@@ -79,6 +79,7 @@ hipError_t launch_pack_sum_merged(const PackArgs& p, const SumArgs& s, hipStream
 hipError_t launch_pipe(const PackArgs& p, const SumArgs& s, hipStream_t st, const Timing* t = nullptr,
                        unsigned long long* pack_relay = nullptr);
 // Most blocks, and vectors per lane, of a grid (or the part of one) that waits for a flag inside the kernel.
+void set_merge_segment(size_t bytes);     // largest payload of ONE merged launch; larger ones go out as several
 void set_gated_tuning(int cap, int unroll);
 // A whole small call (pack, signal, flag poll, sum) in one launch; at most kSmallCallMaxBlocks
 // blocks of 1024 lanes, one 16-byte vector per lane.

@@ -314,6 +314,18 @@ def test_one_gibibyte_calls(orc):
             tbv.stage_peer(b); assert tbv.all_reduce(x)
             torch.cuda.synchronize()
             assert torch.equal(x.view(torch.int32), want.view(torch.int32)), name
+            if name == "bf16":
+                # the peer's payload already in place: four merged launches of 256 MiB each (in place: the fused body)
+                say("1 GiB", name, "early peer")
+                tbv.peer_resident(b)
+                out.zero_()
+                assert tbv.all_reduce(a, out)
+                x = a.clone()
+                assert tbv.all_reduce(x)
+                torch.cuda.synchronize()
+                assert torch.equal(out.view(torch.int32), want.view(torch.int32)), "early peer"
+                assert torch.equal(x.view(torch.int32), want.view(torch.int32)), "early peer, in place"
+                tbv.peer_resident(None)
             del x, out, want
         # 1.5 GiB over the 1 GiB cap: two chunks through the pipeline entry point
         numel = 3 * (n // 4)

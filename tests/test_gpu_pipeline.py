@@ -262,15 +262,18 @@ def test_resident_peer_fused_and_unfused(orc):
             assert not tbv.err()
 
 
-@pytest.mark.parametrize("streaming", [0, 1])
-def test_resident_peer_merged_launch_ragged(orc, streaming):
+@pytest.mark.parametrize("streaming,segment", [(0, 0), (1, 0), (0, 1 << 20)])
+def test_resident_peer_merged_launch_ragged(orc, streaming, segment):
     """Early peer above the one-kernel size: pack blocks and sum blocks share one launch.  Ragged byte counts,
-    three dtypes, in place and out of place, slots reused; the bounce image is read back too."""
+    three dtypes, in place and out of place, slots reused; the bounce image is read back too.  With `segment` the
+    payloads are several segments long, so each call is a row of merged launches of which only the last raises the
+    completion word (what payloads beyond 256 MiB get by default)."""
     import ctypes
     hip = ctypes.CDLL("libamdhip64.so.7")
     hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
     cap = 6 << 20
-    with session(rails=2, cap=cap, TBV_NSLOT=3, TBV_STREAMING=streaming, TBV_UNROLL=(2 if streaming else 0)) as tbv:
+    extra = {"TBV_MERGEMAX": segment} if segment else {}
+    with session(rails=2, cap=cap, TBV_NSLOT=3, TBV_STREAMING=streaming, TBV_UNROLL=(2 if streaming else 0), **extra) as tbv:
         for name in ("bf16", "f16", "f32"):
             dt = DT[name]
             esz = 4 if name == "f32" else 2
@@ -280,7 +283,7 @@ def test_resident_peer_merged_launch_ragged(orc, streaming):
                 a = dev(synth.uniform(71 + k, numel), dt)
                 want = oracle_sum(orc, a, peer[:numel])
                 out = torch.empty_like(a)
-                say("merged", name, numel, "streaming", streaming)
+                say("merged", name, numel, "streaming", streaming, "segment", segment)
                 assert tbv.all_reduce(a, out)
                 torch.cuda.synchronize()
                 assert first_diff(out, want) is None, (name, numel)
