@@ -229,6 +229,123 @@ __global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
     if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
 }
 
+// The whole coded step in one kernel, for a call whose peer image is already in the receive slot: a lane loads its
+// vector of the local tensor once, the lanes of a group agree on min and max, the lane stores its codes (and the
+// group's leader the header) into the bounce slot, decodes them again from its registers (the same fma on the same
+// numbers as a decode of the stored image), decodes the peer's codes of the same elements, adds and stores the
+// output.  Bytes per payload byte of a 2-byte type: read 1, write 0.53, read 0.53, write 1 = 3.06 against 4.6 for
+// the quantise kernel followed by the dequantising sum (which reads this rank's image back), and one launch instead
+// of two.  One vector per lane (blockDim = vectors per superblock: 256, fp32 512), so every load and store of a wave
+// is one contiguous run.  In place is fine: the lane that stores out[i] is the one that loaded a[i].
+// min and max over the LPG (16 or 32) lanes of a group; every lane gets the result.  Within a row of 16 lanes by four
+// rotations on the data-parallel path (no LDS traffic; rotating by 8, 4, 2, 1 and taking the minimum each time leaves
+// every lane with the minimum of all 16, since min and max do not mind an element counted twice); the two rows of an
+// fp32 group then swap through one xor shuffle.
+template <unsigned LPG, bool DPP>
+__device__ __forceinline__ void group_minmax(float& mn, float& mx)
+{
+    if (DPP) {
+#define TBV_ROR(x, n) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + (n), 0xf, 0xf, false))
+        mn = __builtin_fminf(mn, TBV_ROR(mn, 8)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 8));
+        mn = __builtin_fminf(mn, TBV_ROR(mn, 4)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 4));
+        mn = __builtin_fminf(mn, TBV_ROR(mn, 2)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 2));
+        mn = __builtin_fminf(mn, TBV_ROR(mn, 1)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 1));
+#undef TBV_ROR
+        if (LPG == 32) {
+            mn = __builtin_fminf(mn, __shfl_xor(mn, 16, 64));
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, 16, 64));
+        }
+    } else {
+#pragma unroll
+        for (unsigned off = LPG / 2; off >= 1; off >>= 1) {
+            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+        }
+    }
+}
+
+// What a lane holds of one superblock between its loads and its work.
+struct CodedIn { u32x4 v; LaneCodes cb; bool have; };
+
+template <int DT>
+__device__ __forceinline__ CodedIn coded_load(const StepArgs& g, size_t sb, size_t nsb, size_t nvec)
+{
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;
+    CodedIn in;
+    const size_t i = sb * blockDim.x + threadIdx.x;
+    in.have = sb < nsb && i < nvec;
+    const u32x4 zero = {0, 0, 0, 0};
+    in.v = in.have ? g.a[i] : zero;
+    in.cb = LaneCodes{};
+    if (in.have) in.cb = load_codes<EPV>((const unsigned char*)g.b + sb * kCodecSuperBytes, threadIdx.x, LPG);
+    return in;
+}
+
+template <int DT, bool DPP>
+__device__ __forceinline__ void coded_work(const StepArgs& g, size_t sb, const CodedIn& in)
+{
+    constexpr int EPV = Vec<DT>::EPV;
+    constexpr unsigned LPG = kCodecGroup / EPV;             // lanes per group: 16, fp32 32
+    const unsigned tid = threadIdx.x;
+    float f[EPV];
+    Vec<DT>::unpack(in.v, f);
+    float mn = __builtin_inff(), mx = -__builtin_inff();
+    if (in.have) {
+#pragma unroll
+        for (int e = 0; e < EPV; e++) { mn = __builtin_fminf(mn, f[e]); mx = __builtin_fmaxf(mx, f[e]); }
+    }
+    group_minmax<LPG, DPP>(mn, mx);
+    const bool group_has = mn <= mx;                   // false when every lane of the group is past the end
+    mn += 0.0f;                                        // a minimum of -0 is stored as +0
+    const float range = mx - mn;
+    const float scale = !group_has ? 0.0f : (range > 0.0f ? range / 255.0f : 1.0f);
+    const float inv = (group_has && range > 0.0f) ? 255.0f / range : 0.0f;
+    if (!group_has) mn = 0.0f;
+    unsigned char* sbp = (unsigned char*)g.bounce + sb * kCodecSuperBytes;
+    if ((tid % LPG) == 0) {
+        f32x2 hdr = {scale, mn};
+        *(f32x2*)(sbp + (tid / LPG) * 8) = hdr;
+    }
+    // rint first, so the conversion below meets whole numbers only (exact in any rounding mode); it saturates to
+    // 0...255 and drops each code into its byte of the dword
+    uint32_t c[2] = {0, 0};
+#pragma unroll
+    for (int e = 0; e < EPV; e++)
+        c[e / 4] = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf((f[e] - mn) * inv), e % 4, c[e / 4]);
+    if (!in.have) { c[0] = 0; c[1] = 0; }
+    if (EPV == 8) { uint2 cv = {c[0], c[1]}; *(uint2*)(sbp + kSbHeader + (size_t)tid * 8) = cv; }
+    else *(uint32_t*)(sbp + kSbHeader + (size_t)tid * 4) = c[0];
+    if (in.have) {
+        float x[EPV], y[EPV];
+        LaneCodes own;
+        own.hdr.x = scale; own.hdr.y = mn; own.lo = c[0]; own.hi = c[1];
+        decode_codes<EPV>(own, x);                     // the decode of the image just made, from registers
+        decode_codes<EPV>(in.cb, y);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
+        __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + sb * blockDim.x + tid);
+    }
+}
+
+// (Tried and dropped, 16 MiB bf16 cold, 12.65 us as it stands: two superblocks' loads issued together 13.05; the next
+// superblock's loads issued ahead of the work on the current one, with and without a branch around the loads, 13.7-14.1.
+// Taking the parts out one at a time says where the time goes: header stores 0.2 us, code stores 1.4, the peer's codes
+// 1.2, decode + sum + output store 2.8, and 7.3 us remain for reading the local tensor and making the codes.)
+template <int DT, bool DPP>
+__global__ __launch_bounds__(512) void k_coded_step(StepArgs g)
+{
+    constexpr int EPV = Vec<DT>::EPV;
+    const unsigned tid = threadIdx.x;
+    if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
+    if (g.fp && blockIdx.x == 0 && tid == 0) store_sys(g.fp + FP_PACK, g.seq);
+    const size_t nvec = g.nbytes >> 4;
+    const size_t nsb = (nvec * EPV + kCodecSuper - 1) / kCodecSuper;
+    for (size_t sb = blockIdx.x; sb < nsb; sb += gridDim.x) coded_work<DT, DPP>(g, sb, coded_load<DT>(g, sb, nsb, nvec));
+    if (g.cflag) grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, g.sigmode);
+    if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
+}
+
 inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
 template <typename A>
@@ -242,6 +359,7 @@ hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st, const
 // Measured with 16 MiB bf16, cache-cold (quantise / dequantising sum, us): 2048 blocks 7.3 / 8.1, 1024 blocks 7.1 / 7.9,
 // 512 blocks 8.4 / 9.4; two or four passes' loads issued together (U = 2, 4): 7.5 / 8.4 and 7.9 / 9.0, so U stays 1.
 int g_codec_grid_cap = 1024;
+int g_coded_grid_cap = 1024;          // the one-launch coded step (measured: 768 blocks 12.9 us, 1024 and 1536 12.65, 2048 12.75, 4096 13.3)
 
 
 // spb = superblocks one block takes per iteration
@@ -255,7 +373,11 @@ int codec_grid(size_t nbytes, int dtype, bool gated, size_t spb)
 
 }  // namespace
 
-void set_codec_grid_cap(int cap) { g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 1024; }
+void set_codec_grid_cap(int cap)
+{
+    g_codec_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 1024;
+    g_coded_grid_cap = cap >= 1 ? (cap > 8128 ? 8128 : cap) : 1024;
+}
 
 size_t codec_image_bytes(size_t nbytes, int dtype)
 {
@@ -296,6 +418,32 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
         case 0: return launch1(k_sum_quant<0, 1>, grid, 512, st, t, s);
         case 1: return launch1(k_sum_quant<1, 1>, grid, 256, st, t, s);
         default: return launch1(k_sum_quant<2, 1>, grid, 256, st, t, s);
+    }
+}
+
+// The coded step in one launch (see k_coded_step): quantise p.src into the image at p.dst and write
+// out = T(decode(that image) + decode(the received image q.b)).  No gate: for calls whose peer image is in place.
+hipError_t launch_coded_step(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t)
+{
+    if (!p.dst || !p.src || !q.out || !q.b || p.src != q.a || p.nbytes != q.nbytes || (p.nbytes & 15) || p.tagp || q.wait_flag ||
+        !al16(p.dst) || !al16(p.src) || !al16(q.out) || !al16(q.b) || q.dtype < 0 || q.dtype > 2 || (p.cflag && !p.arrive) ||
+        (q.done && !q.done_arrive))
+        return hipErrorInvalidValue;
+    // an output that overlaps the local tensor without being it would be stored over vectors other lanes have yet to load
+    const uintptr_t lo = (uintptr_t)p.src, oo = (uintptr_t)q.out;
+    if (oo != lo && oo < lo + p.nbytes && lo < oo + p.nbytes) return hipErrorInvalidValue;
+    StepArgs s{};
+    s.bounce = (u32x4*)p.dst; s.cflag = p.cflag; s.pack_arrive = p.arrive; s.sigmode = p.sigmode;
+    s.a = (const u32x4*)p.src; s.b = (const u32x4*)q.b; s.out = (u32x4*)q.out; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp;
+    s.done = q.done; s.done_arrive = q.done_arrive;
+    s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
+    const size_t epv = q.dtype == 0 ? 4 : 8, nsb = ((p.nbytes >> 4) * epv + kCodecSuper - 1) / kCodecSuper;
+    const size_t cap = (size_t)g_coded_grid_cap;
+    const int grid = (int)(nsb < 1 ? 1 : nsb < cap ? nsb : cap);
+    switch (q.dtype) {
+        case 0: return launch1(k_coded_step<0, true>, grid, 512, st, t, s);
+        case 1: return launch1(k_coded_step<1, true>, grid, 256, st, t, s);
+        default: return launch1(k_coded_step<2, true>, grid, 256, st, t, s);
     }
 }
 

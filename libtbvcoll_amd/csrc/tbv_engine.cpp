@@ -436,12 +436,16 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             // gate, sum launch).  In place, the sum blocks also wait for the last pack block.
             const bool staged_one = G.staged_merge && G.merge && (!in_place_already || gate_resident) && !one_kernel && plain && G.can_wait_value && G.packsig == 0 &&
                                     !nm && !hold && nbytes <= G.merge_max && (!overlap || inplace);
+            // With the int8 codec and the peer's image already in place: quantise, decode both images and sum in one
+            // kernel that reads the local tensor once and never reads its own image back.
+            const bool coded_one = c->codec && G.merge && in_place_already && !gate_resident && sum_out && G.packsig == 0 && !hold &&
+                                   (!overlap || inplace);
             // Deferred signal: counting the pack's blocks costs about 1.5 us at the end of the kernel.
             // When the next kernel on the stream is one of ours and will not wait behind a stream gate
             // (payload already there, or the flag is polled inside the sum kernel), the pack leaves its
             // completion word alone and that next kernel raises it first thing.
             const bool will_poll_in_kernel = nbytes <= G.fusewait_max;
-            c->deferred = G.defer && !can_fuse && !can_merge && !one_kernel && !staged_one && !G.tag && G.kwait != 1 && G.can_wait_value &&
+            c->deferred = G.defer && !can_fuse && !can_merge && !one_kernel && !staged_one && !coded_one && !G.tag && G.kwait != 1 && G.can_wait_value &&
                           !(G.railsum && c->R > 1) && (c->resident || will_poll_in_kernel);
             pa.pre = take_pending(st);
             // test hook: this call's pack never raises its completion word
@@ -450,7 +454,7 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 pa.cflag = nullptr;
                 c->deferred = false;
                 if (launch_pack(pa, st) != hipSuccess) FAIL("pack kernel launch failed");
-            } else if (one_kernel || can_fuse || can_merge || staged_one) {
+            } else if (one_kernel || can_fuse || can_merge || staged_one || coded_one) {
                 SumArgs sa{};
                 sa.out = sum_out; sa.a = ptr; sa.b = slot_recv(c->slot); sa.b_uncached = (G.uncached & 2) != 0; sa.nbytes = nbytes; sa.dtype = dtype; sa.seq = c->seq;
                 sa.fp = pa.fp;
@@ -461,11 +465,12 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
                 if (G.probe.load(std::memory_order_relaxed)) { sa.done = doneword(c->slot); sa.done_arrive = done_counters(c->slot); }
                 KTimer kt(1);
                 const double tq = nowt();
-                const hipError_t e = one_kernel ? (nm ? launch_row_norm(2, &pa, sa, *nm, st, kt.get()) : launch_small_call(pa, sa, st, kt.get()))
+                const hipError_t e = coded_one ? launch_coded_step(pa, sa, st, kt.get())
+                                   : one_kernel ? (nm ? launch_row_norm(2, &pa, sa, *nm, st, kt.get()) : launch_small_call(pa, sa, st, kt.get()))
                                    : staged_one ? launch_pipe(pa, sa, st, kt.get(), relay_word(c->slot) + 1)
                                    : can_fuse ? launch_pack_sum(pa, sa, st, kt.get()) : launch_pack_sum_merged(pa, sa, st, kt.get());
                 if (e != hipSuccess)
-                    FAIL("%s launch failed: %s (%zu B)", one_kernel ? "one-kernel call" : staged_one ? "pack + gated sum kernel" : "pack+sum kernel",
+                    FAIL("%s launch failed: %s (%zu B)", coded_one ? "coded step" : one_kernel ? "one-kernel call" : staged_one ? "pack + gated sum kernel" : "pack+sum kernel",
                          hipGetErrorName(e), nbytes);
                 G.t_post += nowt() - tq;                       // the launch that carries the sum
                 c->fused = true;

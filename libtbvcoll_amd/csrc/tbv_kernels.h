@@ -117,6 +117,8 @@ size_t codec_image_bytes(size_t nbytes, int dtype);
 void set_codec_grid_cap(int cap);                      // most blocks of a codec launch (0 = default)
 hipError_t launch_quant(const PackArgs& a, int dtype, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum_quant(const SumArgs& s, hipStream_t st, const Timing* t = nullptr);
+// Quantise + dequantising sum of one call in a single launch (peer image already in place; p.src == q.a is the local tensor).
+hipError_t launch_coded_step(const PackArgs& p, const SumArgs& q, hipStream_t st, const Timing* t = nullptr);
 
 // Looks up this device's copy of the built-in counter array of tbv_step_noalloc (once per device).
 bool noalloc_bind_device();

@@ -240,3 +240,67 @@ def test_allreduce_with_codec(mode):
         assert np.array_equal(bits(out), oracle.q8_sum(2, wa, wb, a.numel()))
         tbv.peer_resident(None)
         assert not tbv.err()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("one_launch", [1, 0])
+def test_coded_step_with_the_peer_image_in_place(one_launch):
+    """Early peer with the codec: by default the whole coded step is one kernel (quantise, decode both images, sum)
+    that never reads its own image back; with TBV_MERGE=0 it is the quantise kernel followed by the dequantising
+    sum.  Both must give the oracle's image in the bounce slot and the oracle's sum, out of place and in place,
+    for sizes that end inside a superblock and inside a group."""
+    import ctypes
+    from gpu_util import say, session
+    hip = ctypes.CDLL("libamdhip64.so.7")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    with session(rails=2, cap=8 << 20, TBV_CODEC=1, TBV_CODEC_MIN=64 << 10, TBV_MERGE=one_launch, TBV_NSLOT=3) as tbv:
+        k = 0
+        for name in ("bf16", "f16", "f32"):
+            dt, code = DTS[name]
+            esz = 4 if name == "f32" else 2
+            # whole superblocks; a last superblock of 3 vectors; a last group of one vector; the cap
+            for nb in (1 << 20, (1 << 20) + 48, (256 << 10) + 4096 + 16, 8 << 20):
+                n = nb // esz
+                k += 1
+                a = torch.from_numpy(synth.normal(120 + k, n) * 0.02).to(dt); b = torch.from_numpy(synth.normal(160 + k, n) * 0.02).to(dt)
+                A, B = a.cuda(), b.cuda()
+                wa, wb = oracle.q8_encode(code, bits(a)), oracle.q8_encode(code, bits(b))
+                want = oracle.q8_sum(code, wa, wb, n)
+                tbv.peer_resident(B)
+                for rep in range(4):                               # every ring slot, and one of them twice
+                    out = torch.zeros_like(A)
+                    say("coded step", "one launch" if one_launch else "two launches", name, nb, "rep", rep)
+                    assert tbv.all_reduce(A, out)
+                    torch.cuda.synchronize()
+                    assert np.array_equal(bits(out), want), (name, nb, rep)
+                    img = torch.empty(wa.size, dtype=torch.uint8, device="cuda")
+                    assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), wa.size, 3) == 0
+                    assert np.array_equal(img.cpu().numpy(), wa), (name, nb, rep, "image")
+                x = A.clone()
+                assert tbv.all_reduce(x)                           # in place
+                torch.cuda.synchronize()
+                assert np.array_equal(bits(x), want), (name, nb, "in place")
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), wa.size, 3) == 0
+                assert np.array_equal(img.cpu().numpy(), wa), (name, nb, "image of the in-place call")
+                tbv.peer_resident(None)
+        # hand-made groups: min 0 and max 255 make the step exactly 1, so k + 0.5 lands on a rounding tie (to even) for
+        # every k; a second kind of group holds a huge pair of values, which pushes everything else to the middle code
+        ties = np.concatenate([[0.0, 255.0], np.arange(126) + 0.5]).astype(np.float32)
+        spike = np.concatenate([[-1.0e38, 1.0e38], np.linspace(-1, 1, 126)]).astype(np.float32)
+        pat = np.concatenate([ties, spike, ties[::-1], -ties])
+        a = torch.from_numpy(np.tile(pat, 128)).to(torch.bfloat16); b = torch.from_numpy(np.tile(pat[::-1].copy(), 128)).to(torch.bfloat16)
+        A, B = a.cuda(), b.cuda()
+        wa, wb = oracle.q8_encode(2, bits(a)), oracle.q8_encode(2, bits(b))
+        codes = wa[128:128 + 128]                                  # first group's codes: 0, 255, then the ties
+        assert list(codes[:6]) == [0, 255, 0, 2, 2, 4], list(codes[:8])
+        tbv.peer_resident(B)
+        out = torch.zeros_like(A)
+        say("coded step, hand-made groups")
+        assert tbv.all_reduce(A, out)
+        torch.cuda.synchronize()
+        img = torch.empty(wa.size, dtype=torch.uint8, device="cuda")
+        assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 3), wa.size, 3) == 0
+        assert np.array_equal(img.cpu().numpy(), wa), "image of the hand-made groups"
+        assert np.array_equal(bits(out), oracle.q8_sum(2, wa, wb, a.numel())), "sum of the hand-made groups"
+        tbv.peer_resident(None)
+        assert not tbv.err()

@@ -311,7 +311,10 @@ def test_resident_peer_merged_launch_ragged(orc, streaming, segment):
         assert not tbv.err()
 
 
-@pytest.mark.parametrize("env", [{}, {"TBV_GATEDGRID": 1024, "TBV_GATEDUNROLL": 2}, {"TBV_STREAMING": 1}, {"TBV_STAGEDMERGE": 0}])
+# (the two block sizes: waiting blocks are capped in waves, so wider blocks must not take the wave slots that the
+# deposit kernel, whose completion raises the flag, needs)
+@pytest.mark.parametrize("env", [{}, {"TBV_GATEDGRID": 1024, "TBV_GATEDUNROLL": 2}, {"TBV_STREAMING": 1}, {"TBV_STAGEDMERGE": 0},
+                                 {"TBV_BLOCK": 512}, {"TBV_BLOCK": 1024}])
 def test_staged_call_in_one_launch(orc, env):
     """The peer's payload is not there when the call is made and the call is above the one-kernel size: pack blocks
     and gated sum blocks share one launch.  Ragged sizes, three dtypes, out of place and in place (the sum blocks
