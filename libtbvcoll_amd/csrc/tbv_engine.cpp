@@ -350,6 +350,7 @@ int configure(const char* devs, size_t cap)
     if (G.R < 1 || G.R > MAXRAIL) FAIL("rail count %d out of range 1..%d", G.R, MAXRAIL);
     G.merge = geti("TBV_MERGE", 1);
     G.merge_max = getz("TBV_MERGEMAX", (size_t)256 << 20);
+    if (G.merge_max < ((size_t)1 << 20)) G.merge_max = (size_t)1 << 20;      // segments of a merged launch: whole MiB at least
     set_merge_segment(G.merge_max);
     // a call whose peer payload has not arrived yet, above the one-kernel size: pack blocks + gated sum blocks in one launch
     G.staged_merge = geti("TBV_STAGEDMERGE", 1);
