@@ -34,6 +34,7 @@ from HBM and not from the 256 MB Infinity Cache.  Prints ONE JSON line that also
 """
 import argparse
 import ctypes
+import gc
 import json
 import os
 import re
@@ -153,9 +154,13 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     torch.cuda.synchronize()
     # the last of the warm-up has the shape of the timed region (drained stream, a short burst, drained again): the
     # first such region after a long queue of launches runs 10-15 % slower than the ones that follow it
+    # (nothing stands between it and the timed region: a pause of even 20 us before a region costs its first launch
+    # 4-9 us, the progress threads having gone to sleep and the GPU idle)
+    tbv.stats4()                       # drop what the warm-up (and the first call's stream probe) accumulated
+    gc.collect()
+    gc.disable()                       # no collector pause inside a region of a few hundred microseconds
     for _ in range(2):
         timed(min(steps, 48))
-    tbv.stats4()                       # drop what the warm-up (and the first call's stream probe) accumulated
     wall = timed(steps)
     if not fit_region:
         # a comparison leg (not the headline, whose K steps are timed exactly once): best of three regions, so that a
@@ -214,6 +219,7 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     torch.cuda.synchronize()
     err = tbv.err()
     tbv.shutdown()
+    gc.enable()
     for k, _ in env:
         os.environ.pop(k, None)
     return {"wall": wall, "steps": steps, "long_wall": long_wall, "long_steps": long_steps, "ok": ok and not err, "enq_us": enq,

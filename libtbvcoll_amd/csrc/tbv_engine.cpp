@@ -497,7 +497,10 @@ int enqueue_pack(const void* ptr, void* sum_out, size_t nbytes, int dtype, hipSt
             x.q[h % G.nslot] = Item{c->seq, c->slot, nbytes, c->R, c->xbytes, peer, c->resident, c->host_wire};
             x.q_head.store(h + 1, std::memory_order_seq_cst);
         }
-        for (int r = 0; r < c->R; r++) wake_if(G.rr[r].napping, &G.cv_item);
+        // the rails sleep on one condition variable: one broadcast wakes all of them (a wake is a system call, and the
+        // first call after an idle spell pays it on the caller's thread)
+        for (int r = 0; r < c->R; r++)
+            if (G.rr[r].napping.load(std::memory_order_seq_cst)) { wake_if(G.rr[r].napping, &G.cv_item); break; }
     } else {
         // synchronous mode: the caller thread does everything (step4/libtbvcoll.cpp:482-493)
         if (hipMemcpyAsync(slot_send(c->slot), ptr, nbytes, hipMemcpyDeviceToDevice, st) != hipSuccess) FAIL("copy into send slot failed");
