@@ -140,12 +140,18 @@ static constexpr unsigned kGroup = 32;
 static constexpr unsigned kCtrLine = 16;       // words per counter line (64 bytes)
 
 // Returns true in thread 0 of the block that found itself the last one (false everywhere else).
+//
+// `keep` (mode 0 only; block-uniform): the wave's last `keep` memory operations are stores that need not be counted
+// (a fused body's output stores, issued after all of its bounce stores).  A wave's memory operations complete in the
+// order they were issued, so waiting until only `keep` are outstanding has seen every counted store acknowledged.
 __device__ __forceinline__ bool grid_complete(unsigned long long* word, unsigned long long seq,
-                                              unsigned int* ctr, unsigned int bid, unsigned int nblk, int mode)
+                                              unsigned int* ctr, unsigned int bid, unsigned int nblk, int mode, int keep = 0)
 {
     bool was_last = false;
     if (mode == 2) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (mode == 0 && keep == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else if (mode == 0 && keep == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         if (mode == 1) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
