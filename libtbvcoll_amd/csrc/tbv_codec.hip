@@ -223,7 +223,7 @@ __global__ __launch_bounds__(512) void k_sum_quant(StepArgs g)
             decode_codes<EPV>(cb[u], y);
 #pragma unroll
             for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
-            __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + (sb0 + u) * blockDim.x + tid);
+            st_result(g.out + (sb0 + u) * blockDim.x + tid, Vec<DT>::pack(x), g.out_through);
         }
     }
     if (g.done) grid_complete(g.done, g.seq, g.done_arrive, blockIdx.x, gridDim.x, 1);
@@ -324,7 +324,7 @@ __device__ __forceinline__ void coded_work(const StepArgs& g, size_t sb, const C
         decode_codes<EPV>(in.cb, y);
 #pragma unroll
         for (int e = 0; e < EPV; e++) x[e] = x[e] + y[e];
-        __builtin_nontemporal_store(Vec<DT>::pack(x), g.out + sb * blockDim.x + tid);
+        st_result(g.out + sb * blockDim.x + tid, Vec<DT>::pack(x), g.out_through);
     }
 }
 
@@ -413,6 +413,7 @@ hipError_t launch_sum_quant(const SumArgs& q, hipStream_t st, const Timing* t)
     s.wait_flag = q.wait_flag; s.relay = q.relay; s.spin_limit = q.spin_limit_ticks; s.b_uncached = q.b_uncached;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.pre_word = q.pre.word; s.pre_seq = q.pre.seq;
+    s.out_through = streaming_profile();
     const int grid = codec_grid(q.nbytes, q.dtype, q.wait_flag != nullptr, 1);
     switch (q.dtype) {
         case 0: return launch1(k_sum_quant<0, 1>, grid, 512, st, t, s);
@@ -437,6 +438,7 @@ hipError_t launch_coded_step(const PackArgs& p, const SumArgs& q, hipStream_t st
     s.a = (const u32x4*)p.src; s.b = (const u32x4*)q.b; s.out = (u32x4*)q.out; s.nbytes = p.nbytes; s.seq = p.seq; s.fp = p.fp;
     s.done = q.done; s.done_arrive = q.done_arrive;
     s.pre_word = p.pre.word; s.pre_seq = p.pre.seq;
+    s.out_through = streaming_profile();
     const size_t epv = q.dtype == 0 ? 4 : 8, nsb = ((p.nbytes >> 4) * epv + kCodecSuper - 1) / kCodecSuper;
     const size_t cap = (size_t)g_coded_grid_cap;
     const int grid = (int)(nsb < 1 ? 1 : nsb < cap ? nsb : cap);

@@ -40,9 +40,26 @@ template <bool STREAM> __device__ __forceinline__ uint32_t __attribute__((ext_ve
 {
     return STREAM ? __builtin_nontemporal_load(p) : *p;
 }
+// The output in the streaming profile is written THROUGH the L2 (system scope) as well as non-temporally: a line
+// that is merely non-temporal still sits dirty in the L2 until it is evicted or the kernel ends, where the
+// write-back of what is left stands between this kernel and the next (merged launch, 16 MiB cache-cold, same
+// box: non-temporal 12.20 us per launch, write-through + non-temporal 11.89, write-through alone 12.65,
+// plain 13.0).  No builtin sets the scope bits of a 16-byte store, hence the instruction itself; it has no
+// result, so the compiler's wait counting is at most conservative about it.
+__device__ __forceinline__ void st_through(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" :: "v"(p), "v"(v) : "memory");
+}
 template <bool STREAM> __device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {
-    __builtin_nontemporal_store(v, p);
+    if (STREAM) st_through(p, v);
+    else __builtin_nontemporal_store(v, p);
+}
+// The same choice at run time (block-uniform), for the kernels that are not compiled once per profile.
+__device__ __forceinline__ void st_result(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v, int through)
+{
+    if (through) st_through(p, v);
+    else __builtin_nontemporal_store(v, p);
 }
 template <bool STREAM> __device__ __forceinline__ void st_bounce(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {
@@ -262,6 +279,7 @@ struct StepArgs {
                                       // the same launch waits for it (beside its flag) when the output aliases the local tensor
     int b_uncached;             // the received payload lies in uncached memory: the gate needs no cache invalidation
     unsigned tiles;             // sum part of a pipeline launch: tiles of blockDim x US vectors, taken in turn by its blocks
+    int out_through;            // codec kernels: results are written through the L2 (streaming profile)
 };
 
 }  // namespace tbv

@@ -62,6 +62,7 @@ int sum_grid(size_t nbytes, int dtype);
 // block (0 = defaults), and the cache-hint profile (0 = operands stay cache resident, 1 = streaming from HBM).
 // Every call sets all four.
 void set_tuning(int unroll, int grid_cap, int block, int streaming);
+bool streaming_profile();       // the cache-hint profile set_tuning was last given
 
 hipError_t launch_pack(const PackArgs& a, hipStream_t st, const Timing* t = nullptr);
 hipError_t launch_sum(const SumArgs& a, hipStream_t st, const Timing* t = nullptr);

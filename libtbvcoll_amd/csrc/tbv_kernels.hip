@@ -405,6 +405,8 @@ void set_tuning(int unroll, int grid_cap, int block, int streaming)
     g_stream = streaming != 0;
 }
 
+bool streaming_profile() { return g_stream; }
+
 static inline bool al16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
 // One launch of a kernel that takes a single argument struct; with `t` the

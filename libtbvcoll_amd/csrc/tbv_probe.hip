@@ -26,7 +26,12 @@ constexpr int kBlock = 256;
 //                           copy  plain 4/stride 5.6, non-temporal both 4/stride 6.0, non-temporal load 1/pass 6.47
 // kind 0: read (the xor of what was read is kept so the loads cannot be dropped)   kind 1: write
 // kind 2: copy, non-temporal loads   kind 3: copy, plain accesses
-template <int KIND, int U, bool NT_LOAD, bool LOOP>
+// WT: stores written through the L2 and non-temporal (what the data path's streaming profile does with its output)
+__device__ __forceinline__ void store_through(u32x4* p, u32x4 v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" :: "v"(p), "v"(v) : "memory");
+}
+template <int KIND, int U, bool NT_LOAD, bool LOOP, bool WT = false>
 __global__ __launch_bounds__(kBlock) void k_stream(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t nvec, u32x4* sink)
 {
     const size_t tile = (size_t)kBlock * U;
@@ -45,6 +50,7 @@ __global__ __launch_bounds__(kBlock) void k_stream(const u32x4* __restrict__ src
             const size_t i = base + (size_t)u * kBlock + threadIdx.x;
             if (i >= nvec) continue;
             if (KIND == 0) { acc.x ^= x[u].x; acc.y ^= x[u].y; acc.z ^= x[u].z; acc.w ^= x[u].w; }
+            else if (WT) store_through(dst + i, x[u]);
             else dst[i] = x[u];
         }
         if (!LOOP) break;
@@ -53,7 +59,8 @@ __global__ __launch_bounds__(kBlock) void k_stream(const u32x4* __restrict__ src
 }
 
 // The four streams of one all-reduce step and nothing else: read the local tensor and the received payload, write
-// the bounce and the bf16 sum, two vectors per lane, one pass, no block counting, no completion word, no gate.  What
+// the bounce and the bf16 sum (with the data path's own cache hints), two vectors per lane, one pass, no block
+// counting, no completion word, no gate.  What
 // the memory system delivers to this body on cache-cold operands is the floor under every form of the step.
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void k_step_floor(const u32x4* a, const u32
         if (i >= nvec) continue;
         u32x4 r = {add_bf16x2(x[u].x, y[u].x), add_bf16x2(x[u].y, y[u].y), add_bf16x2(x[u].z, y[u].z), add_bf16x2(x[u].w, y[u].w)};
         __builtin_nontemporal_store(x[u], bounce + i);
-        __builtin_nontemporal_store(r, out + i);
+        store_through(out + i, r);
     }
 }
 
@@ -98,10 +105,24 @@ struct Bufs {
     }
 };
 
-// shape 0: four vectors per lane, grid-stride, at most `cap` blocks; shape 1: one vector per lane, one pass
+// shape 0: four vectors per lane, grid-stride, at most `cap` blocks; shape 1: one vector per lane, one pass;
+// shapes 2 and 3: the same two with stores written through the L2 (write and non-temporal copy only)
 void launch(int kind, int shape, size_t cap, hipStream_t st, hipEvent_t e0, hipEvent_t e1, const char* src, char* dst, size_t nvec, u32x4* sink)
 {
     const u32x4* s = (const u32x4*)src; u32x4* d = (u32x4*)dst;
+    if (shape == 3) {
+        const dim3 grid((unsigned)((nvec + kBlock - 1) / kBlock));
+        if (kind == 1) hipExtLaunchKernelGGL((k_stream<1, 1, false, false, true>), grid, dim3(kBlock), 0, st, e0, e1, 0, s, d, nvec, sink);
+        else hipExtLaunchKernelGGL((k_stream<2, 1, true, false, true>), grid, dim3(kBlock), 0, st, e0, e1, 0, s, d, nvec, sink);
+        return;
+    }
+    if (shape == 2) {
+        const size_t tiles4 = (nvec + (size_t)kBlock * 4 - 1) / ((size_t)kBlock * 4);
+        const dim3 grid((unsigned)std::min(tiles4, cap));
+        if (kind == 1) hipExtLaunchKernelGGL((k_stream<1, 4, false, true, true>), grid, dim3(kBlock), 0, st, e0, e1, 0, s, d, nvec, sink);
+        else hipExtLaunchKernelGGL((k_stream<2, 4, true, true, true>), grid, dim3(kBlock), 0, st, e0, e1, 0, s, d, nvec, sink);
+        return;
+    }
     if (shape == 1) {
         const dim3 grid((unsigned)((nvec + kBlock - 1) / kBlock));
         switch (kind) {
@@ -147,9 +168,10 @@ extern "C" int tbv_emu_hbm_probe(int kind, size_t bytes, size_t pool_bytes, int 
     const size_t cap = bytes >= ((size_t)256 << 20) ? 16384 : 1024;
     int rc = 0;
     double sum = 0, mn = 1e30;
-    // both shapes, the faster one (by its mean) is the figure: which one wins depends on the kind and the size
-    for (int shape = 0; shape < 2 && rc == 0; shape++) {
+    // every shape, the fastest one (by its mean) is the figure: which one wins depends on the kind and the size
+    for (int shape = 0; shape < 4 && rc == 0; shape++) {
         if (kind == 3 && shape == 1) break;                // the plain copy stays the one plain shape, as a reference
+        if (shape >= 2 && kind != 1 && kind != 2) break;   // only kinds that store have write-through shapes
         for (int i = 0; i < 3 + reps && rc == 0; i++) {    // three untimed launches first
             const size_t w = ((size_t)i % windows) * bytes;
             const bool timed = i >= 3;
