@@ -47,13 +47,15 @@ void timed_wait(pthread_cond_t* cv)          // caller holds G.mx; naps at most 
 // `napping` flag before it re-checks its condition under G.mx, and the waker publishes the
 // condition before it reads the flag (both sequentially consistent), so one of the two always
 // sees the other; a nap is 2 ms at most in any case.
+// The broadcast comes after the mutex has been released again: taking it once is what orders this wake against a
+// waiter between its re-check and its wait, and the woken threads then do not run into a mutex the waker still holds.
 void wake_if(std::atomic<int>& napping, pthread_cond_t* cv)
 {
     std::atomic_thread_fence(std::memory_order_seq_cst);
     if (!napping.load(std::memory_order_seq_cst)) return;
     pthread_mutex_lock(&G.mx);
-    pthread_cond_broadcast(cv);
     pthread_mutex_unlock(&G.mx);
+    pthread_cond_broadcast(cv);
 }
 
 inline bool queue_empty(const Rail& x)
@@ -130,8 +132,15 @@ void* progress_rail(void* arg)
     bool owns[MAXSLOT];
     while (G.run.load(std::memory_order_acquire)) {
         if (queue_empty(x)) {
+            // Spin, then sleep.  The reference spins 30 us (step4/libtbvcoll.cpp:54,236-243); a caller that makes a call
+            // every few hundred microseconds then finds the thread asleep every time and pays a wake (a system call,
+            // and now and then 20-50 us when the woken thread is placed on the caller's core) on its own thread at the
+            // start of each burst.  So while the recent gaps between items have been short, the thread spins through
+            // gaps of up to twice their smoothed length; sparse callers get the reference's 30 us.
             const double ts = nowt();
-            while (nowt() - ts < SPIN_US * 1e-6 && queue_empty(x) && G.run.load(std::memory_order_relaxed)) { }
+            double spin = G.spin_us;
+            if (x.gap_us > 0 && 2 * x.gap_us <= G.spin_max_us && 2 * x.gap_us > spin) spin = 2 * x.gap_us;
+            while (nowt() - ts < spin * 1e-6 && queue_empty(x) && G.run.load(std::memory_order_relaxed)) { }
             if (queue_empty(x)) {
                 pthread_mutex_lock(&G.mx);
                 x.napping.store(1, std::memory_order_seq_cst);
@@ -141,6 +150,10 @@ void* progress_rail(void* arg)
             }
             if (!G.run.load(std::memory_order_relaxed)) break;
             if (queue_empty(x)) continue;
+            // (a gap counts as TBV_SPINMAX at most: one long pause of a busy caller does not send the threads to sleep
+            // for its next several bursts, and a sparse caller's gaps settle at the cap, beyond the spinning range)
+            const double gap = std::min((nowt() - ts) * 1e6, G.spin_max_us);
+            x.gap_us = x.gap_us > 0 ? 0.75 * x.gap_us + 0.25 * gap : gap;
         }
         const uint64_t tail = x.q_tail.load(std::memory_order_relaxed);
         const uint64_t head = x.q_head.load(std::memory_order_acquire);
@@ -329,6 +342,8 @@ int configure(const char* devs, size_t cap)
     G.rail1max = getz("TBV_RAIL1MAX", 96u * 1024u);
     G.cpu = geti("TBV_CPU", -1);
     { const char* e = getenv("TBV_WDOG"); G.wdog = (e && atof(e) > 0) ? atof(e) : 10.0; }
+    { const char* e = getenv("TBV_SPIN"); G.spin_us = (e && atof(e) >= 0) ? atof(e) : SPIN_US; }
+    { const char* e = getenv("TBV_SPINMAX"); G.spin_max_us = (e && atof(e) >= 0) ? atof(e) : 1000.0; }
     G.tag = (geti("TBV_TAG", 0) && G.async && G.gpusig) ? 1 : 0;
     // bit 0: send ring uncached (the reference's default, step4/libtbvcoll.cpp:314); bit 1: receive ring uncached, the
     // kind of memory a peer's writes land in (costs the sum nothing: 12.9 us per 16 MiB step either way)
@@ -690,7 +705,7 @@ int init_impl(int rank, const char* devs, const char* peer_ip, int port, size_t 
     }
     for (int r = 0; r < G.R; r++) {
         Rail& x = G.rr[r];
-        x.idx = r; x.q_head.store(0); x.q_tail.store(0); x.script_pos = 0; x.napping.store(0);
+        x.idx = r; x.q_head.store(0); x.q_tail.store(0); x.script_pos = 0; x.napping.store(0); x.gap_us = 0;
         x.rl_post = x.rl_arr = 0; x.rl_n = 0;
         if (hipStreamCreateWithFlags(&x.wire, hipStreamNonBlocking) != hipSuccess) FAIL("side stream creation failed");
     }

@@ -55,6 +55,7 @@ struct Rail {
     Item q[MAXSLOT];
     std::atomic<uint64_t> q_head{0}, q_tail{0};
     std::atomic<int> napping{0};              // the progress thread is (about to be) asleep on cv_item
+    double gap_us = 0;                        // recent idle gaps between items, smoothed (progress thread only)
     pthread_t th{};
     bool started = false;
     hipStream_t wire = nullptr;               // side stream that plays the peer's writes
@@ -88,6 +89,8 @@ struct Engine {
     size_t codec_min = (size_t)512 << 10;     // TBV_CODEC_MIN
     size_t cap = 0, stride = 0, rail1max = 96u * 1024u, chunkb = 0, fusewait_max = 0;
     double wdog = 10.0;
+    double spin_us = SPIN_US;                 // how long a progress thread spins on an empty queue before it sleeps (TBV_SPIN)
+    double spin_max_us = 1000.0;              // while calls keep coming at gaps of up to half of this, the threads spin through the gaps (TBV_SPINMAX; 0 = never)
     double tick_hz = 1e8;                     // rate of the constant clock the kernels bound their waits with
     int can_wait_value = 1, can_write_value = 1;
     // memory
