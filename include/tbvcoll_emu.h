@@ -134,7 +134,8 @@ int tbv_emu_run_quant(void* image, const void* src, size_t nbytes, int dtype, vo
 int tbv_emu_run_sum_quant(void* out, const void* own_image, const void* recv_image, size_t nbytes, int dtype, void* stream);
 
 /* Standalone row kernel for benches and tests: mode 0: normed = rmsnorm(a) * weight;
- * mode 1: out = a + b, normed = rmsnorm(out) * weight. */
+ * mode 1: out = a + b, normed = rmsnorm(out) * weight.  mode + 4: the operands are cache-cold (buffers beyond
+ * the caches, read once): the hints the engine takes in its streaming profile.  Same bits either way. */
 int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const void* b, void* normed, const void* weight, float eps,
                          size_t rows, size_t hidden, int dtype, void* stream);
 

@@ -313,7 +313,7 @@ extern "C" int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, con
     ONE_CALLER();
     hipStream_t st = (hipStream_t)stream;
     note_stream(stream, nbytes);
-    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
+    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows, G.streaming};
     const double te = nowt();
     Call c{};
     if (enqueue_pack(ptr, outp, nbytes, dtype, st, &c, &nm) != 0) return -1;
@@ -323,15 +323,18 @@ extern "C" int tbv_ar_allreduce_rmsnorm(void* ptr, void* outp, void* normed, con
     return 0;
 }
 
-// Standalone row kernel for benches and tests: mode 0 normalises `a`; mode 1 writes out = a + b and normalises it.
+// Standalone row kernel for benches and tests: mode 0 normalises `a`; mode 1 writes out = a + b and normalises it;
+// + 4: the operands are cache-cold (what the engine derives from its ring size: the streaming profile's hints).
 extern "C" int tbv_emu_run_sum_norm(int mode, void* out, const void* a, const void* b, void* normed, const void* weight, float eps,
                                     size_t rows, size_t hidden, int dtype, void* stream)
 {
+    const int cold = (mode & 4) ? 1 : 0;
+    if (mode >= 0) mode &= 3;
     if (dtype < 0 || dtype > 2 || mode < 0 || mode > 1 || !row_norm_shape_ok(rows, hidden, dtype)) return -1;
     const size_t esz = dtype == 0 ? 4 : 2;
     SumArgs sa{};
     sa.out = out; sa.a = a; sa.b = b; sa.nbytes = rows * hidden * esz; sa.dtype = dtype;
-    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows};
+    NormArgs nm{weight, normed, eps, (unsigned)(hidden * esz / 16), (unsigned)rows, cold};
     return launch_row_norm(mode, nullptr, sa, nm, (hipStream_t)stream) == hipSuccess ? 0 : -1;
 }
 

@@ -101,6 +101,7 @@ struct NormArgs {
     float eps;
     unsigned row_vecs;
     unsigned rows;
+    int cold = 0;               // host side only: the operands come from HBM, not from a cache (streaming profile)
 };
 static constexpr int kRowNormMaxVecs = 4096;          // 64 KiB per row: 1024 lanes x 4 vectors
 static constexpr int kRowNormMaxSmallRows = 128;      // one-launch form: every block must be resident while it waits

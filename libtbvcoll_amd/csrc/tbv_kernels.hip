@@ -83,7 +83,7 @@ __device__ __forceinline__ void step_body(const StepArgs& g, unsigned bid, unsig
 }
 
 template <int DT, int U, bool PACK, bool SUM, bool STREAM>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
+__global__ __launch_bounds__(kMaxSmallThreads, (U <= 2 ? 8 : 1)) void k_step(StepArgs g)
 {
     const unsigned tid = threadIdx.x;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);     // deferred signal of the kernel before
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_step(StepArgs g)
 // while its output stores are still on their way (16 MiB cache-cold: 13.9 us with every block counted after
 // all of its stores, four vectors per lane, 1024 blocks -> 12.8 us this way with two vectors per lane, one pass).
 template <int DT, int U, bool STREAM>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_fused(StepArgs g)
+__global__ __launch_bounds__(kMaxSmallThreads, 8) void k_fused(StepArgs g)
 {
     const unsigned tid = threadIdx.x, nthr = blockDim.x, bid = blockIdx.x;
     if (g.pre_word && bid == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_fused(StepArgs g)
 // is served by that XCD's L2 (counters: 4.007 bytes per payload byte cross the fabric).
 // Only legal when the received payload is already in place: there is no gate in this kernel.
 template <int DT, int UP, int US, bool STREAM>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_merged(StepArgs g)
+__global__ __launch_bounds__(kMaxSmallThreads, ((UP <= 2 && US <= 2) ? 8 : 1)) void k_merged(StepArgs g)
 {
     const unsigned tid = threadIdx.x, P = g.pack_blocks;
     if (g.pre_word && blockIdx.x == 0 && tid == 0) store_sys(g.pre_word, g.pre_seq);
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(kMaxSmallThreads) void k_merged(StepArgs g)
 //                      the sum blocks also wait for the last pack block (sm.pack_relay), since a sum block may
 //                      otherwise store out[i] while a pack block has yet to read a[i].
 template <int DT, int UP, int US, bool STREAM>
-__global__ __launch_bounds__(kMaxSmallThreads) void k_pipe(StepArgs pk, StepArgs sm)
+__global__ __launch_bounds__(kMaxSmallThreads, ((UP <= 2 && US <= 2) ? 8 : 1)) void k_pipe(StepArgs pk, StepArgs sm)
 {
     const unsigned tid = threadIdx.x, P = pk.pack_blocks;
     if (pk.pre_word && blockIdx.x == 0 && tid == 0) store_sys(pk.pre_word, pk.pre_seq);

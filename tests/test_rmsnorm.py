@@ -129,6 +129,11 @@ def test_row_kernel_bit_exact_vs_oracle(name, rows, hidden):
     assert lib.tbv_emu_run_sum_norm(0, None, out.data_ptr(), None, n2.data_ptr(), W.data_ptr(), 1e-6, rows, hidden, code, st) == 0
     torch.cuda.synchronize()
     assert np.array_equal(bits(n2), want_normed)
+    # the cache-cold variant of the looping form (mode + 4: non-temporal loads) computes the same bits
+    o3 = torch.empty_like(A); n3 = torch.empty_like(A)
+    assert lib.tbv_emu_run_sum_norm(1 + 4, o3.data_ptr(), A.data_ptr(), B.data_ptr(), n3.data_ptr(), W.data_ptr(), 1e-6, rows, hidden, code, st) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(o3), want_out) and np.array_equal(bits(n3), want_normed)
     # and torch's own formula on the GPU agrees to 2 ulp
     d = ulp_distance(normed.cpu(), torch_rmsnorm(out, W, 1e-6).cpu(), dt)
     assert int(d.max()) <= (8 if name == "f32" else 2)
