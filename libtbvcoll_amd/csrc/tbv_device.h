@@ -44,11 +44,20 @@ template <bool STREAM> __device__ __forceinline__ uint32_t __attribute__((ext_ve
 // that is merely non-temporal still sits dirty in the L2 until it is evicted or the kernel ends, where the
 // write-back of what is left stands between this kernel and the next (merged launch, 16 MiB cache-cold, same
 // box: non-temporal 12.20 us per launch, write-through + non-temporal 11.89, write-through alone 12.65,
-// plain 13.0).  No builtin sets the scope bits of a 16-byte store, hence the instruction itself; it has no
-// result, so the compiler's wait counting is at most conservative about it.
+// plain 13.0).  No builtin sets the scope bits of a 16-byte global store; the raw buffer store takes them as its
+// cache-policy operand (sc0 = 1, nt = 2, sc1 = 16), so the store goes out as a buffer store whose descriptor is
+// built around the wave's lowest address (lanes store to ascending addresses, so the first active lane holds it;
+// a wave's stores span far less than the 4 GiB a 32-bit offset reaches).  An inline-asm store is not an option:
+// the compiler does not know it for a 16-byte store and leaves out the wait states this GPU needs before the
+// next instruction may overwrite the data registers (seen as stale first dwords in some vectors).
 __device__ __forceinline__ void st_through(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" :: "v"(p), "v"(v) : "memory");
+    const uint64_t addr = (uint64_t)p;
+    // (the builtin returns a signed int: through uint32_t, or a low word with bit 31 set would smear over the high one)
+    const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32)) << 32) |
+                          (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)addr);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffff, 0x00020000);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (uint32_t)(addr - base), 0, 1 | 2 | 16);
 }
 template <bool STREAM> __device__ __forceinline__ void st_out(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v)
 {

@@ -181,6 +181,93 @@ __global__ __launch_bounds__(kMaxSmallThreads, ((UP <= 2 && US <= 2) ? 8 : 1)) v
     }
 }
 
+// The same launch for the common case, stripped: a payload of whole tiles that one pass covers (every
+// [rows x hidden] tensor whose size is a multiple of 8 KiB, up to the counters' 8128 blocks per half), no
+// diagnostics, no deferred signal of an earlier kernel, no done word.  The general kernel carries 208 bytes of
+// arguments, four conditional stores and a bounds-checked loop for all of that; without them the 16 MiB cold
+// launch is 0.3 us shorter (replicas on one box: 11.87 us lean, 12.05 with the general kernel's arguments and
+// conditional stores, 12.21 with its loop and bounds as well; the general kernel itself 12.15).
+struct WholeArgs {
+    const u32x4* a; const u32x4* b; u32x4* bounce; u32x4* out;
+    unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long seq; unsigned pack_blocks;
+};
+template <int DT, int U, bool STREAM>
+__global__ __launch_bounds__(kThreads) void k_merged_whole(WholeArgs g)
+{
+    const unsigned tid = threadIdx.x, P = g.pack_blocks;
+    if (blockIdx.x < P) {
+        const u32x4* a = g.a + (size_t)blockIdx.x * (kThreads * U) + tid;
+        u32x4* d = g.bounce + (size_t)blockIdx.x * (kThreads * U) + tid;
+        u32x4 x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + u * kThreads);
+#pragma unroll
+        for (int u = 0; u < U; u++) st_bounce<STREAM>(d + u * kThreads, x[u]);
+        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, P, 0);
+    } else {
+        const size_t base = (size_t)(blockIdx.x - P) * (kThreads * U) + tid;
+        u32x4 x[U], y[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+#pragma unroll
+        for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+    }
+}
+
+// The fused body and the staged launch for the same common case (whole tiles of two vectors per lane, no
+// diagnostics, no done word, no earlier kernel's signal).
+template <int DT, bool STREAM>
+__global__ __launch_bounds__(kThreads) void k_fused_whole(WholeArgs g)
+{
+    constexpr int U = 2;
+    const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+    u32x4 x[U], y[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, true>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+#pragma unroll
+    for (int u = 0; u < U; u++) st_bounce<STREAM>(g.bounce + base + u * kThreads, x[u]);
+    asm volatile("" ::: "memory");      // the output stores stay behind the bounce stores
+#pragma unroll
+    for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+    grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, 0, U);
+}
+
+struct WholeGateArgs {
+    WholeArgs w;
+    const unsigned long long* wait_flag; unsigned long long* relay; unsigned long long spin_limit;
+    unsigned tiles;             // tiles of the sum part, taken in turn by its blocks
+};
+// (the received payload lies in uncached memory: the gate needs no cache invalidation; the host checks that)
+template <int DT, bool STREAM>
+__global__ __launch_bounds__(kThreads) void k_pipe_whole(WholeGateArgs q)
+{
+    constexpr int U = 2;
+    const WholeArgs& g = q.w;
+    const unsigned tid = threadIdx.x, P = g.pack_blocks;
+    if (blockIdx.x < P) {
+        if (blockIdx.x == 0 && tid == 0 && __hip_atomic_load(q.wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= g.seq)
+            __hip_atomic_store(q.relay, g.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);       // one look, as in k_pipe
+        const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
+        u32x4 x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads);
+#pragma unroll
+        for (int u = 0; u < U; u++) st_bounce<STREAM>(g.bounce + base + u * kThreads, x[u]);
+        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, P, 0);
+    } else {
+        const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
+        gate_wait_as(bid, q.wait_flag, g.seq, q.spin_limit, q.relay, nullptr, false, nullptr, true);
+        for (unsigned t = bid; t < q.tiles; t += S) {
+            const size_t base = (size_t)t * (kThreads * U) + tid;
+            u32x4 x[U], y[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+#pragma unroll
+            for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+        }
+    }
+}
+
 // ---------------------------------------------------------------- the pipeline step
 //
 // Pack blocks and GATED sum blocks in one launch, each set with its own arguments.  Blocks [0, P) pack and raise
@@ -533,6 +620,23 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
     // can count the blocks), completion counted on the bounce stores alone
     Geom g = geom_for(p.nbytes, false, true);
     if (g.unroll != 2) g.unroll = 1;
+    // whole tiles, one pass, nothing but the step itself: the stripped kernel
+    if (g.unroll == 2 && g.block == kThreads && !(s.nbytes & 15) && (s.nbytes >> 4) == (size_t)g.grid * kThreads * 2 &&
+        s.cflag && !s.pre_word && !s.fp && !s.tagp && !s.done) {
+        const WholeArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid};
+        if (g_stream) {
+            switch (q.dtype) {
+                case 0: return launch1(k_fused_whole<0, true>, g.grid, kThreads, st, t, w);
+                case 1: return launch1(k_fused_whole<1, true>, g.grid, kThreads, st, t, w);
+                default: return launch1(k_fused_whole<2, true>, g.grid, kThreads, st, t, w);
+            }
+        }
+        switch (q.dtype) {
+            case 0: return launch1(k_fused_whole<0, false>, g.grid, kThreads, st, t, w);
+            case 1: return launch1(k_fused_whole<1, false>, g.grid, kThreads, st, t, w);
+            default: return launch1(k_fused_whole<2, false>, g.grid, kThreads, st, t, w);
+        }
+    }
     if (g_stream) {
         switch (q.dtype) {
             case 0: return launch_fused_u<0, true>(s, g, st, t);
@@ -557,11 +661,35 @@ static hipError_t launch_merged_u(const StepArgs& s, int grid, int block, int un
     }
 }
 
+template <int DT, bool STREAM>
+static hipError_t launch_merged_whole(const WholeArgs& w, int grid, int unroll, hipStream_t st, const Timing* t)
+{
+    if (unroll == 2) return launch1(k_merged_whole<DT, 2, STREAM>, grid, kThreads, st, t, w);
+    return launch1(k_merged_whole<DT, 1, STREAM>, grid, kThreads, st, t, w);
+}
+
 static hipError_t launch_merged_one(int dtype, StepArgs& s, hipStream_t st, const Timing* t)
 {
     const Geom g = geom_for(s.nbytes, false, true);
     s.pack_blocks = (unsigned)g.grid;
     const int grid = 2 * g.grid, u = g.unroll == 8 ? 4 : g.unroll;
+    // whole tiles, one pass, nothing but the step itself: the stripped kernel
+    if ((u == 1 || u == 2) && g.block == kThreads && !(s.nbytes & 15) && (s.nbytes >> 4) == (size_t)g.grid * kThreads * u &&
+        s.cflag && s.sigmode == 0 && !s.pre_word && !s.fp && !s.tagp && !s.done) {
+        const WholeArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid};
+        if (g_stream) {
+            switch (dtype) {
+                case 0: return launch_merged_whole<0, true>(w, grid, u, st, t);
+                case 1: return launch_merged_whole<1, true>(w, grid, u, st, t);
+                default: return launch_merged_whole<2, true>(w, grid, u, st, t);
+            }
+        }
+        switch (dtype) {
+            case 0: return launch_merged_whole<0, false>(w, grid, u, st, t);
+            case 1: return launch_merged_whole<1, false>(w, grid, u, st, t);
+            default: return launch_merged_whole<2, false>(w, grid, u, st, t);
+        }
+    }
     if (g_stream) {
         switch (dtype) {
             case 0: return launch_merged_u<0, true>(s, grid, g.block, u, st, t);
@@ -664,6 +792,24 @@ hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, cons
     const int S = (int)(T < wcap ? T : wcap);
     sm.tiles = (unsigned)T;
     pk.pack_blocks = (unsigned)P;
+    // one staged call of whole tiles, out of place, nothing but the step itself: the stripped kernel
+    if (p.src == q.a && p.nbytes == q.nbytes && !same && q.wait_flag && q.b_uncached && up == 2 && us == 2 && block == kThreads &&
+        !(p.nbytes & 15) && pvec == (size_t)P * kThreads * 2 && !p.pre.word && !q.pre.word && !q.fp && !q.done && !p.fp) {
+        const WholeGateArgs w{WholeArgs{pk.a, sm.b, pk.bounce, sm.out, pk.cflag, pk.pack_arrive, pk.seq, (unsigned)P},
+                              q.wait_flag, q.relay, q.spin_limit_ticks, (unsigned)T};
+        if (g_stream) {
+            switch (q.dtype) {
+                case 0: return launch1(k_pipe_whole<0, true>, P + S, kThreads, st, t, w);
+                case 1: return launch1(k_pipe_whole<1, true>, P + S, kThreads, st, t, w);
+                default: return launch1(k_pipe_whole<2, true>, P + S, kThreads, st, t, w);
+            }
+        }
+        switch (q.dtype) {
+            case 0: return launch1(k_pipe_whole<0, false>, P + S, kThreads, st, t, w);
+            case 1: return launch1(k_pipe_whole<1, false>, P + S, kThreads, st, t, w);
+            default: return launch1(k_pipe_whole<2, false>, P + S, kThreads, st, t, w);
+        }
+    }
     if (g_stream) {
         switch (q.dtype) {
             case 0: return launch_pipe_u<0, true>(up, us, P + S, block, st, t, pk, sm);

@@ -29,7 +29,12 @@ constexpr int kBlock = 256;
 // WT: stores written through the L2 and non-temporal (what the data path's streaming profile does with its output)
 __device__ __forceinline__ void store_through(u32x4* p, u32x4 v)
 {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" :: "v"(p), "v"(v) : "memory");
+    const uint64_t addr = (uint64_t)p;
+    // (the builtin returns a signed int: through uint32_t, or a low word with bit 31 set would smear over the high one)
+    const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32)) << 32) |
+                          (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)addr);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffff, 0x00020000);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (uint32_t)(addr - base), 0, 1 | 2 | 16);     // sc0 nt sc1
 }
 template <int KIND, int U, bool NT_LOAD, bool LOOP, bool WT = false>
 __global__ __launch_bounds__(kBlock) void k_stream(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t nvec, u32x4* sink)
