@@ -187,49 +187,55 @@ __global__ __launch_bounds__(kMaxSmallThreads, ((UP <= 2 && US <= 2) ? 8 : 1)) v
 // arguments, four conditional stores and a bounds-checked loop for all of that; without them the 16 MiB cold
 // launch is 0.3 us shorter (replicas on one box: 11.87 us lean, 12.05 with the general kernel's arguments and
 // conditional stores, 12.21 with its loop and bounds as well; the general kernel itself 12.15).
+// Their arguments are separate kernel parameters, the ones a wave needs first in front: this file is compiled with
+// kernel-argument preloading, which hands the first 14 dwords of scalar and pointer parameters to every wave in
+// registers at launch instead of having it load them (a structure passed by value is not preloaded).  A wave of
+// these kernels lives about 5 us, and the load of its arguments stood in front of its first data load: the same
+// lean launch measures 11.85 us with its arguments loaded and 11.59 us with them preloaded.
 struct WholeArgs {
     const u32x4* a; const u32x4* b; u32x4* bounce; u32x4* out;
     unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long seq; unsigned pack_blocks;
 };
 template <int DT, int U, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_merged_whole(WholeArgs g)
+__global__ __launch_bounds__(kThreads) void k_merged_whole(unsigned P, const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
+                                                           unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq)
 {
-    const unsigned tid = threadIdx.x, P = g.pack_blocks;
+    const unsigned tid = threadIdx.x;
     if (blockIdx.x < P) {
-        const u32x4* a = g.a + (size_t)blockIdx.x * (kThreads * U) + tid;
-        u32x4* d = g.bounce + (size_t)blockIdx.x * (kThreads * U) + tid;
+        const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
         u32x4 x[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + u * kThreads);
+        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
 #pragma unroll
-        for (int u = 0; u < U; u++) st_bounce<STREAM>(d + u * kThreads, x[u]);
-        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, P, 0);
+        for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+        grid_complete(cflag, seq, pack_arrive, blockIdx.x, P, 0);
     } else {
         const size_t base = (size_t)(blockIdx.x - P) * (kThreads * U) + tid;
         u32x4 x[U], y[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+        for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(a + base + u * kThreads); y[u] = ld_b<STREAM>(b + base + u * kThreads); }
 #pragma unroll
-        for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+        for (int u = 0; u < U; u++) st_out<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
     }
 }
 
 // The fused body and the staged launch for the same common case (whole tiles of two vectors per lane, no
 // diagnostics, no done word, no earlier kernel's signal).
 template <int DT, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_fused_whole(WholeArgs g)
+__global__ __launch_bounds__(kThreads) void k_fused_whole(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
+                                                          unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq)
 {
     constexpr int U = 2;
     const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
     u32x4 x[U], y[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, true>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+    for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, true>(a + base + u * kThreads); y[u] = ld_b<STREAM>(b + base + u * kThreads); }
 #pragma unroll
-    for (int u = 0; u < U; u++) st_bounce<STREAM>(g.bounce + base + u * kThreads, x[u]);
+    for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
     asm volatile("" ::: "memory");      // the output stores stay behind the bounce stores
 #pragma unroll
-    for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
-    grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, gridDim.x, 0, U);
+    for (int u = 0; u < U; u++) st_out<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+    grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0, U);
 }
 
 struct WholeGateArgs {
@@ -239,31 +245,32 @@ struct WholeGateArgs {
 };
 // (the received payload lies in uncached memory: the gate needs no cache invalidation; the host checks that)
 template <int DT, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_pipe_whole(WholeGateArgs q)
+__global__ __launch_bounds__(kThreads) void k_pipe_whole(unsigned P, const u32x4* a, const u32x4* b, u32x4* out, unsigned long long* relay,
+                                                         unsigned long long seq, u32x4* bounce, const unsigned long long* wait_flag,
+                                                         unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long spin_limit, unsigned tiles)
 {
     constexpr int U = 2;
-    const WholeArgs& g = q.w;
-    const unsigned tid = threadIdx.x, P = g.pack_blocks;
+    const unsigned tid = threadIdx.x;
     if (blockIdx.x < P) {
-        if (blockIdx.x == 0 && tid == 0 && __hip_atomic_load(q.wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= g.seq)
-            __hip_atomic_store(q.relay, g.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);       // one look, as in k_pipe
+        if (blockIdx.x == 0 && tid == 0 && __hip_atomic_load(wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= seq)
+            __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);       // one look, as in k_pipe
         const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
         u32x4 x[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads);
+        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
 #pragma unroll
-        for (int u = 0; u < U; u++) st_bounce<STREAM>(g.bounce + base + u * kThreads, x[u]);
-        grid_complete(g.cflag, g.seq, g.pack_arrive, blockIdx.x, P, 0);
+        for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+        grid_complete(cflag, seq, pack_arrive, blockIdx.x, P, 0);
     } else {
         const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
-        gate_wait_as(bid, q.wait_flag, g.seq, q.spin_limit, q.relay, nullptr, false, nullptr, true);
-        for (unsigned t = bid; t < q.tiles; t += S) {
+        gate_wait_as(bid, wait_flag, seq, spin_limit, relay, nullptr, false, nullptr, true);
+        for (unsigned t = bid; t < tiles; t += S) {
             const size_t base = (size_t)t * (kThreads * U) + tid;
             u32x4 x[U], y[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(g.a + base + u * kThreads); y[u] = ld_b<STREAM>(g.b + base + u * kThreads); }
+            for (int u = 0; u < U; u++) { x[u] = ld_a<STREAM, false>(a + base + u * kThreads); y[u] = ld_b<STREAM>(b + base + u * kThreads); }
 #pragma unroll
-            for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+            for (int u = 0; u < U; u++) st_out<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
         }
     }
 }
@@ -506,6 +513,15 @@ static hipError_t launch1(void (*kernel)(A), int grid, int block, hipStream_t st
     return hipGetLastError();
 }
 
+// The same for a kernel that takes its arguments one by one.
+template <typename... P, typename... A>
+static hipError_t launch_each(void (*kernel)(P...), int grid, int block, hipStream_t st, const Timing* t, A... args)
+{
+    if (t && t->start && t->stop) hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, t->start, t->stop, 0, static_cast<P>(args)...);
+    else hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, st, static_cast<P>(args)...);
+    return hipGetLastError();
+}
+
 template <int DT, bool PACK, bool SUM, bool STREAM>
 static hipError_t launch_step_u(const StepArgs& s, const Geom& g, hipStream_t st, const Timing* t)
 {
@@ -626,15 +642,15 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
         const WholeArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid};
         if (g_stream) {
             switch (q.dtype) {
-                case 0: return launch1(k_fused_whole<0, true>, g.grid, kThreads, st, t, w);
-                case 1: return launch1(k_fused_whole<1, true>, g.grid, kThreads, st, t, w);
-                default: return launch1(k_fused_whole<2, true>, g.grid, kThreads, st, t, w);
+                case 0: return launch_each(k_fused_whole<0, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+                case 1: return launch_each(k_fused_whole<1, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+                default: return launch_each(k_fused_whole<2, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
             }
         }
         switch (q.dtype) {
-            case 0: return launch1(k_fused_whole<0, false>, g.grid, kThreads, st, t, w);
-            case 1: return launch1(k_fused_whole<1, false>, g.grid, kThreads, st, t, w);
-            default: return launch1(k_fused_whole<2, false>, g.grid, kThreads, st, t, w);
+            case 0: return launch_each(k_fused_whole<0, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+            case 1: return launch_each(k_fused_whole<1, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+            default: return launch_each(k_fused_whole<2, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
         }
     }
     if (g_stream) {
@@ -664,8 +680,8 @@ static hipError_t launch_merged_u(const StepArgs& s, int grid, int block, int un
 template <int DT, bool STREAM>
 static hipError_t launch_merged_whole(const WholeArgs& w, int grid, int unroll, hipStream_t st, const Timing* t)
 {
-    if (unroll == 2) return launch1(k_merged_whole<DT, 2, STREAM>, grid, kThreads, st, t, w);
-    return launch1(k_merged_whole<DT, 1, STREAM>, grid, kThreads, st, t, w);
+    if (unroll == 2) return launch_each(k_merged_whole<DT, 2, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+    return launch_each(k_merged_whole<DT, 1, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
 }
 
 static hipError_t launch_merged_one(int dtype, StepArgs& s, hipStream_t st, const Timing* t)
@@ -799,15 +815,15 @@ hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, cons
                               q.wait_flag, q.relay, q.spin_limit_ticks, (unsigned)T};
         if (g_stream) {
             switch (q.dtype) {
-                case 0: return launch1(k_pipe_whole<0, true>, P + S, kThreads, st, t, w);
-                case 1: return launch1(k_pipe_whole<1, true>, P + S, kThreads, st, t, w);
-                default: return launch1(k_pipe_whole<2, true>, P + S, kThreads, st, t, w);
+                case 0: return launch_each(k_pipe_whole<0, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+                case 1: return launch_each(k_pipe_whole<1, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+                default: return launch_each(k_pipe_whole<2, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
             }
         }
         switch (q.dtype) {
-            case 0: return launch1(k_pipe_whole<0, false>, P + S, kThreads, st, t, w);
-            case 1: return launch1(k_pipe_whole<1, false>, P + S, kThreads, st, t, w);
-            default: return launch1(k_pipe_whole<2, false>, P + S, kThreads, st, t, w);
+            case 0: return launch_each(k_pipe_whole<0, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+            case 1: return launch_each(k_pipe_whole<1, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+            default: return launch_each(k_pipe_whole<2, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
         }
     }
     if (g_stream) {
