@@ -159,7 +159,7 @@ int tbv_emu_launch_floor(int reps, double* us_per_launch);
  * the uncached bounce and the bf16 sum; no block counting, no completion word, no gate), `reps`
  * launches back to back over 12 rotating local/output tensors and 16 rotating received/bounce
  * buffers that it allocates itself (the uncached ones are kept until the process ends).
- * bytes: multiple of 16, 4 KiB .. 64 MiB.  Returns 0, or -1. */
+ * bytes: whole tiles of 8 KiB, up to 64 MiB.  Returns 0, or -1. */
 int tbv_emu_step_floor(size_t bytes, int reps, double* us_per_launch);
 
 #ifdef __cplusplus

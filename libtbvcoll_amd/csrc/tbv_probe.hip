@@ -77,19 +77,17 @@ __device__ __forceinline__ uint32_t add_bf16x2(uint32_t x, uint32_t y)
     bf16x2 r = __builtin_convertvector(s, bf16x2);
     return __builtin_bit_cast(uint32_t, r);
 }
-__global__ __launch_bounds__(kBlock) void k_step_floor(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out, size_t nvec)
+__global__ __launch_bounds__(kBlock) void k_step_floor(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out)
 {
-    const size_t base = (size_t)blockIdx.x * kBlock * 2;
+    // whole tiles only (the host checks), arguments preloaded into registers (this file's compile flags): nothing
+    // stands between the start of a wave and its first load
+    const size_t base = (size_t)blockIdx.x * kBlock * 2 + threadIdx.x;
     u32x4 x[2], y[2];
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const size_t i = base + (size_t)u * kBlock + threadIdx.x;
-        if (i < nvec) { x[u] = a[i]; y[u] = __builtin_nontemporal_load(b + i); }
-    }
+    for (int u = 0; u < 2; u++) { x[u] = a[base + (size_t)u * kBlock]; y[u] = __builtin_nontemporal_load(b + base + (size_t)u * kBlock); }
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-        const size_t i = base + (size_t)u * kBlock + threadIdx.x;
-        if (i >= nvec) continue;
+        const size_t i = base + (size_t)u * kBlock;
         u32x4 r = {add_bf16x2(x[u].x, y[u].x), add_bf16x2(x[u].y, y[u].y), add_bf16x2(x[u].z, y[u].z), add_bf16x2(x[u].w, y[u].w)};
         __builtin_nontemporal_store(x[u], bounce + i);
         store_through(out + i, r);
@@ -209,7 +207,7 @@ extern "C" int tbv_emu_step_floor(size_t bytes, int reps, double* us_per_launch)
     constexpr int NA = 12, NB = 16;
     static char* bounce_pool = nullptr;
     static size_t bounce_pool_bytes = 0;
-    if (bytes < 4096 || (bytes & 15) || bytes > ((size_t)64 << 20) || reps < 1 || reps > 100000 || !us_per_launch) return -1;
+    if (bytes < 8192 || (bytes & 8191) || bytes > ((size_t)64 << 20) || reps < 1 || reps > 100000 || !us_per_launch) return -1;     // whole tiles of 8 KiB
     if (bounce_pool_bytes < NB * bytes) {
         char* p = nullptr;
         if (hipExtMallocWithFlags((void**)&p, NB * bytes, hipDeviceMallocUncached) != hipSuccess) return -1;
@@ -220,10 +218,10 @@ extern "C" int tbv_emu_step_floor(size_t bytes, int reps, double* us_per_launch)
     hipEvent_t e0 = nullptr, e1 = nullptr;
     int rc = -1;
     const size_t nvec = bytes >> 4;
-    const dim3 grid((unsigned)((nvec + 2 * kBlock - 1) / (2 * kBlock)));
+    const dim3 grid((unsigned)(nvec / (2 * kBlock)));
     auto run = [&](int i) {
         hipLaunchKernelGGL(k_step_floor, grid, dim3(kBlock), 0, st, (const u32x4*)(a + (size_t)(i % NA) * bytes), (const u32x4*)(b + (size_t)(i % NB) * bytes),
-                           (u32x4*)(bounce_pool + (size_t)(i % NB) * bytes), (u32x4*)(o + (size_t)(i % NA) * bytes), nvec);
+                           (u32x4*)(bounce_pool + (size_t)(i % NB) * bytes), (u32x4*)(o + (size_t)(i % NA) * bytes));
     };
     if (hipMalloc((void**)&a, NA * bytes) == hipSuccess && hipMalloc((void**)&o, NA * bytes) == hipSuccess &&
         hipMalloc((void**)&b, NB * bytes) == hipSuccess && hipMemset(a, 0x3c, NA * bytes) == hipSuccess &&
