@@ -93,11 +93,14 @@ def own_warmup(warmup, nslot, nbuf):
     return max(warmup, 2 * math.lcm(nslot, nbuf), 48)
 
 
-def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0, check="exact", staged=False, fit_region=False):
+def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_steps=0, check="exact", staged=False, fit_region=False,
+                inplace=False):
     """`steps` timed calls after `warmup` untimed ones (never fewer than two turns of every rotating tensor and
     ring slot, so no buffer is touched for the first time inside the clock), then an optional long run, then a
     pass of the same steps with the dispatch timestamps of every kernel launch.  With `staged` the peer's payload
-    is handed to the emulated wire before every call instead of sitting in the receive slots beforehand."""
+    is handed to the emulated wire before every call instead of sitting in the receive slots beforehand.  With
+    `inplace` every call overwrites its local tensor (the reference's outp == NULL); the rotating tensors then
+    accumulate, and exactness is checked on a last round of calls from fresh copies."""
     n = N_PREFILL
     for k in TUNING_KEYS:
         os.environ.pop(k, None)
@@ -113,6 +116,9 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     fn = tbv.raw_fn()
     ps = ctypes.c_void_p(st.cuda_stream)
     ptrs = [(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(o.data_ptr())) for x, o in zip(locs, outs)]
+    if inplace:
+        locs[0] = a.clone()            # `a` itself stays intact for the check
+        ptrs = [(ctypes.c_void_p(x.data_ptr()), None) for x in locs]
     if not staged:
         tbv.peer_resident(b)           # the peer's payload sits in every receive slot before the clock starts
     stage, pb = tbv.lib().tbv_emu_stage_peer, ctypes.c_void_p(b.data_ptr())
@@ -196,6 +202,15 @@ def run_prefill(tbv, torch, synth, st, steps, warmup, nslot, nbuf, env=(), long_
     torch.cuda.synchronize()           # the averages are per completed transfer: let all of them complete
     enq = tbv.stats4()[3]
     want = a + b
+    if inplace:
+        # repeated sums of small numbers stay finite; for the check every tensor starts again from `a`
+        torch.cuda.synchronize()
+        for x in locs:
+            x.copy_(a)
+        for _ in range(nbuf):
+            step()
+        torch.cuda.synchronize()
+        outs = locs
     if check == "codec":
         # with the int8 codec every element is within half a quantisation step of each operand's group of 128
         # (step = (max - min) / 255), plus the rounding of the result to bf16
@@ -669,6 +684,18 @@ def main():
 
     if "fused" in legs and not fused_headline:
         leg("fused", leg_fused)
+
+    def leg_inplace():
+        r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, inplace=True)
+        rms = r["wall"] / sub_steps * 1e3
+        line["cold_in_place"] = {"what": "the same cache-cold step in place (the reference's outp == NULL: the output is the local tensor). "
+                                         "Library default: the fused body (one lane loads a vector once and does both stores), 4N", "steps": sub_steps,
+                                 "ms_per_step": round(rms, 5), "value": round(4 * n / (rms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                                 "frac_of_peak": round(4 * n / (rms * 1e-3) / HBM_PEAK, 4), "bit_exact": r["ok"],
+                                 "kernel": kernel_roofline(4 * n, r["sum_us"], r["sum_min_us"], r["n_sum"], ceiling)}
+
+    if "fused" in legs:
+        leg("inplace", leg_inplace)
 
     def leg_staged():
         r = run_prefill(tbv, torch, synth, st, sub_steps, args.warmup, COLD_NSLOT, COLD_NBUF, staged=True)

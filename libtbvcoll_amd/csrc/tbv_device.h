@@ -64,6 +64,16 @@ template <bool STREAM> __device__ __forceinline__ void st_out(uint32_t __attribu
     if (STREAM) st_through(p, v);
     else __builtin_nontemporal_store(v, p);
 }
+// In place the output's lines are in the L2 already (this kernel has just read them as the local tensor), and writing
+// them through costs more than it saves: fused body, 16 MiB cache-cold in place, 13.4 us written through, 12.2
+// non-temporal or plain.  `in_place` is uniform over the grid.
+// (A merged launch for in-place calls, its pack and sum waves ordered pairwise through a word per wave, was built
+// and measured: 12.1 us, no better than the fused body with these stores, so in place keeps the fused body.)
+template <bool STREAM> __device__ __forceinline__ void st_out_at(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v, bool in_place)
+{
+    if (STREAM && !in_place) st_through(p, v);
+    else __builtin_nontemporal_store(v, p);
+}
 // The same choice at run time (block-uniform), for the kernels that are not compiled once per profile.
 __device__ __forceinline__ void st_result(uint32_t __attribute__((ext_vector_type(4)))* p, uint32_t __attribute__((ext_vector_type(4))) v, int through)
 {

@@ -116,6 +116,7 @@ __global__ __launch_bounds__(kMaxSmallThreads, 8) void k_fused(StepArgs g)
     const size_t nvec = g.nbytes >> 4;
     const size_t tile = (size_t)nthr * U;
     bool ordered = true;        // the wave's last U memory operations are output stores (or it has issued none at all)
+    const bool in_place = (const void*)g.out == (const void*)g.a;
     for (size_t base = (size_t)bid * tile; base < nvec; base += (size_t)gridDim.x * tile) {
         u32x4 x[U], y[U];
         if (base + tile <= nvec) {
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(kMaxSmallThreads, 8) void k_fused(StepArgs g)
             for (int u = 0; u < U; u++) st_bounce<STREAM>(g.bounce + base + (size_t)u * nthr + tid, x[u]);
             asm volatile("" ::: "memory");      // the output stores stay behind the bounce stores
 #pragma unroll
-            for (int u = 0; u < U; u++) st_out<STREAM>(g.out + base + (size_t)u * nthr + tid, add_vec<DT>(x[u], y[u]));
+            for (int u = 0; u < U; u++) st_out_at<STREAM>(g.out + base + (size_t)u * nthr + tid, add_vec<DT>(x[u], y[u]), in_place);
             ordered = true;
         } else {
 #pragma unroll
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(kMaxSmallThreads, 8) void k_fused(StepArgs g)
                     x[u] = ld_a<STREAM, true>(g.a + i);
                     y[u] = ld_b<STREAM>(g.b + i);
                     st_bounce<STREAM>(g.bounce + i, x[u]);
-                    st_out<STREAM>(g.out + i, add_vec<DT>(x[u], y[u]));
+                    st_out_at<STREAM>(g.out + i, add_vec<DT>(x[u], y[u]), in_place);
                 }
             }
             ordered = false;
@@ -233,8 +234,9 @@ __global__ __launch_bounds__(kThreads) void k_fused_whole(const u32x4* a, const 
 #pragma unroll
     for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
     asm volatile("" ::: "memory");      // the output stores stay behind the bounce stores
+    const bool in_place = (const void*)out == (const void*)a;
 #pragma unroll
-    for (int u = 0; u < U; u++) st_out<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]));
+    for (int u = 0; u < U; u++) st_out_at<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]), in_place);
     grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0, U);
 }
 

@@ -311,6 +311,54 @@ def test_resident_peer_merged_launch_ragged(orc, streaming, segment):
         assert not tbv.err()
 
 
+@pytest.mark.parametrize("streaming", [0, 1])
+def test_resident_peer_in_place_whole_tiles(orc, streaming):
+    """In place (the reference's outp == NULL) with the peer early and a payload of whole tiles: the stripped fused
+    body (one lane loads a vector once, stores it to the bounce and stores the sum over it).  Every call's output
+    equals the oracle's sum AND its bounce image equals the ORIGINAL tensor; then bursts of back-to-back in-place
+    calls on distinct tensors, checked after each burst."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so.7")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    cap = 16 << 20
+    with session(rails=2, cap=cap, TBV_NSLOT=4, TBV_STREAMING=streaming) as tbv:
+        for name, sizes in (("bf16", (2 << 20, 6 << 20, 8 << 20, 16 << 20)), ("f16", (16 << 20,)), ("f32", (4 << 20, 16 << 20))):
+            dt = DT[name]
+            esz = 4 if name == "f32" else 2
+            peer = dev(synth.uniform(170, cap // esz), dt)
+            tbv.peer_resident(peer)
+            for k, nbytes in enumerate(sizes):
+                numel = nbytes // esz
+                a = dev(synth.uniform(171 + k, numel), dt)
+                want = oracle_sum(orc, a, peer[:numel])
+                img = torch.empty_like(a)
+                for it in range(6):
+                    c = a.clone()
+                    say("in place, whole tiles", name, nbytes, "streaming", streaming, it)
+                    assert tbv.all_reduce(c)
+                    torch.cuda.synchronize()
+                    assert first_diff(c, want) is None, (name, nbytes, it)
+                    assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 4), nbytes, 3) == 0
+                    assert np.array_equal(bits_np(img), bits_np(a)), (name, nbytes, it, "bounce image")
+            tbv.peer_resident(None)
+        # back to back, no synchronisation inside a burst
+        peer = dev(synth.uniform(180, cap // 2), torch.bfloat16)
+        tbv.peer_resident(peer)
+        srcs = [dev(synth.uniform(181 + i, cap // 2), torch.bfloat16) for i in range(6)]
+        wants = [x + peer for x in srcs]
+        work = [x.clone() for x in srcs]
+        say("in place, whole tiles, bursts", streaming)
+        for rnd in range(12):
+            for w in work:
+                assert tbv.all_reduce(w)
+            torch.cuda.synchronize()
+            for x, w, want in zip(srcs, work, wants):
+                assert torch.equal(w.view(torch.int16), want.view(torch.int16)), rnd
+                w.copy_(x)
+        tbv.peer_resident(None)
+        assert not tbv.err()
+
+
 # (the two block sizes: waiting blocks are capped in waves, so wider blocks must not take the wave slots that the
 # deposit kernel, whose completion raises the flag, needs)
 @pytest.mark.parametrize("env", [{}, {"TBV_GATEDGRID": 1024, "TBV_GATEDUNROLL": 2}, {"TBV_STREAMING": 1}, {"TBV_STAGEDMERGE": 0},
