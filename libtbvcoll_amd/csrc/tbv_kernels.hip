@@ -182,35 +182,86 @@ __global__ __launch_bounds__(kMaxSmallThreads, ((UP <= 2 && US <= 2) ? 8 : 1)) v
     }
 }
 
-// The same launch for the common case, stripped: a payload of whole tiles that one pass covers (every
-// [rows x hidden] tensor whose size is a multiple of 8 KiB, up to the counters' 8128 blocks per half), no
-// diagnostics, no deferred signal of an earlier kernel, no done word.  The general kernel carries 208 bytes of
-// arguments, four conditional stores and a bounds-checked loop for all of that; without them the 16 MiB cold
-// launch is 0.3 us shorter (replicas on one box: 11.87 us lean, 12.05 with the general kernel's arguments and
+// The same launch for the common case, stripped: a payload that one pass covers (up to the counters' 8128 blocks
+// per part), default block size, no diagnostics, no deferred signal of an earlier kernel, no done word.  Every block
+// runs straight code on a whole tile; only a block among the last eight of its part looks at the byte count at all
+// (tile_kind below).  The general kernel carries 208 bytes of arguments, four conditional stores and a
+// bounds-checked loop; without them the 16 MiB cold launch is 0.3 us shorter (replicas on one box: 11.87 us lean, 12.05 with the general kernel's arguments and
 // conditional stores, 12.21 with its loop and bounds as well; the general kernel itself 12.15).
 // Their arguments are separate kernel parameters, the ones a wave needs first in front: this file is compiled with
 // kernel-argument preloading, which hands the first 14 dwords of scalar and pointer parameters to every wave in
 // registers at launch instead of having it load them (a structure passed by value is not preloaded).  A wave of
 // these kernels lives about 5 us, and the load of its arguments stood in front of its first data load: the same
 // lean launch measures 11.85 us with its arguments loaded and 11.59 us with them preloaded.
-struct WholeArgs {
+struct LeanArgs {
     const u32x4* a; const u32x4* b; u32x4* bounce; u32x4* out;
     unsigned long long* cflag; unsigned int* pack_arrive; unsigned long long seq; unsigned pack_blocks;
+    size_t nbytes;
 };
+// A payload that is not a whole number of tiles ends in a ragged one: its vectors are bounds-checked and the bytes past
+// the last whole vector follow, all by the one block that owns that tile (the last of its part of the grid).  Every
+// other block runs the straight code; `nbytes` is looked at by the last block only.
+// The parts of these grids are a multiple of eight blocks long, so that the pack block and the sum block of a tile
+// always land on the same XCD (12 MiB + 2 bytes, 1537 tiles: 10.6 us with 1537 blocks per part, the second read of
+// the local tensor then coming from memory, against 9.7 for 12 MiB).  A block among the last eight of its part finds
+// out what it has: a whole tile (0), the ragged one (1), or nothing at all (2).
+template <int U>
+__device__ __forceinline__ int tile_kind(unsigned t, unsigned P, size_t nbytes)
+{
+    constexpr size_t kTileBytes = (size_t)kThreads * U * 16;
+    if (t + 8 <= P) return 0;
+    const size_t tiles = (nbytes + kTileBytes - 1) / kTileBytes;
+    return t >= tiles ? 2 : (t == tiles - 1 && (nbytes & (kTileBytes - 1))) ? 1 : 0;
+}
+template <int DT, int U, bool STREAM, bool PACK, bool SUM>
+__device__ __forceinline__ void ragged_tile(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out, size_t first_vec, size_t nbytes, bool in_place)
+{
+    const unsigned tid = threadIdx.x;
+    const size_t nvec = nbytes >> 4;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const size_t i = first_vec + (size_t)u * kThreads + tid;
+        if (i < nvec) {
+            const u32x4 x = ld_a<STREAM, PACK && SUM>(a + i);
+            if (PACK) st_bounce<STREAM>(bounce + i, x);
+            if (SUM) st_out_at<STREAM>(out + i, add_vec<DT>(x, ld_b<STREAM>(b + i)), in_place);
+        }
+    }
+    const unsigned tail = (unsigned)(nbytes & 15);
+    if (tail) {
+        const size_t off = nvec << 4;
+        typedef typename Elem<DT>::T T;
+        if (PACK && tid < tail) ((unsigned char*)bounce)[off + tid] = ((const unsigned char*)a)[off + tid];
+        if (SUM) __syncthreads();        // in place: the bytes above are read before any of them is overwritten
+        if (SUM && tid < tail / sizeof(T))
+            ((T*)((char*)out + off))[tid] = Elem<DT>::add(((const T*)((const char*)a + off))[tid], ((const T*)((const char*)b + off))[tid]);
+    }
+}
 template <int DT, int U, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_merged_whole(unsigned P, const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
-                                                           unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq)
+__global__ __launch_bounds__(kThreads) void k_merged_lean(unsigned P, const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
+                                                           unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq,
+                                                           size_t nbytes)
 {
     const unsigned tid = threadIdx.x;
     if (blockIdx.x < P) {
-        const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
-        u32x4 x[U];
+        const int kind = tile_kind<U>(blockIdx.x, P, nbytes);
+        if (kind == 1) {
+            ragged_tile<DT, U, STREAM, true, false>(a, b, bounce, out, (size_t)blockIdx.x * (kThreads * U), nbytes, false);
+        } else if (kind == 0) {
+            const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
+            u32x4 x[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
+            for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
 #pragma unroll
-        for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+            for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+        }
         grid_complete(cflag, seq, pack_arrive, blockIdx.x, P, 0);
-    } else {
+        return;
+    }
+    const int kind = tile_kind<U>(blockIdx.x - P, P, nbytes);
+    if (kind == 1) {
+        ragged_tile<DT, U, STREAM, false, true>(a, b, bounce, out, (size_t)(blockIdx.x - P) * (kThreads * U), nbytes, false);
+    } else if (kind == 0) {
         const size_t base = (size_t)(blockIdx.x - P) * (kThreads * U) + tid;
         u32x4 x[U], y[U];
 #pragma unroll
@@ -220,13 +271,20 @@ __global__ __launch_bounds__(kThreads) void k_merged_whole(unsigned P, const u32
     }
 }
 
-// The fused body and the staged launch for the same common case (whole tiles of two vectors per lane, no
+// The fused body and the staged launch for the same common case (one pass of tiles of two vectors per lane, no
 // diagnostics, no done word, no earlier kernel's signal).
 template <int DT, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_fused_whole(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
-                                                          unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq)
+__global__ __launch_bounds__(kThreads) void k_fused_lean(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
+                                                          unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq,
+                                                          size_t nbytes)
 {
     constexpr int U = 2;
+    constexpr size_t kTileBytes = (size_t)kThreads * U * 16;
+    if (blockIdx.x == gridDim.x - 1 && (nbytes & (kTileBytes - 1))) {
+        ragged_tile<DT, U, STREAM, true, true>(a, b, bounce, out, (size_t)blockIdx.x * (kThreads * U), nbytes, (const void*)out == (const void*)a);
+        grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0);
+        return;
+    }
     const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
     u32x4 x[U], y[U];
 #pragma unroll
@@ -240,33 +298,44 @@ __global__ __launch_bounds__(kThreads) void k_fused_whole(const u32x4* a, const 
     grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0, U);
 }
 
-struct WholeGateArgs {
-    WholeArgs w;
+struct LeanGateArgs {
+    LeanArgs w;
     const unsigned long long* wait_flag; unsigned long long* relay; unsigned long long spin_limit;
     unsigned tiles;             // tiles of the sum part, taken in turn by its blocks
 };
 // (the received payload lies in uncached memory: the gate needs no cache invalidation; the host checks that)
 template <int DT, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_pipe_whole(unsigned P, const u32x4* a, const u32x4* b, u32x4* out, unsigned long long* relay,
+__global__ __launch_bounds__(kThreads) void k_pipe_lean(unsigned P, const u32x4* a, const u32x4* b, u32x4* out, unsigned long long* relay,
                                                          unsigned long long seq, u32x4* bounce, const unsigned long long* wait_flag,
-                                                         unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long spin_limit, unsigned tiles)
+                                                         unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long spin_limit, unsigned tiles,
+                                                         size_t nbytes)
 {
     constexpr int U = 2;
+    constexpr size_t kTileBytes = (size_t)kThreads * U * 16;
     const unsigned tid = threadIdx.x;
     if (blockIdx.x < P) {
         if (blockIdx.x == 0 && tid == 0 && __hip_atomic_load(wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= seq)
             __hip_atomic_store(relay, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);       // one look, as in k_pipe
-        const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
-        u32x4 x[U];
+        const int kind = tile_kind<U>(blockIdx.x, P, nbytes);
+        if (kind == 1) {
+            ragged_tile<DT, U, STREAM, true, false>(a, b, bounce, out, (size_t)blockIdx.x * (kThreads * U), nbytes, false);
+        } else if (kind == 0) {
+            const size_t base = (size_t)blockIdx.x * (kThreads * U) + tid;
+            u32x4 x[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
+            for (int u = 0; u < U; u++) x[u] = ld_a<STREAM, false>(a + base + u * kThreads);
 #pragma unroll
-        for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+            for (int u = 0; u < U; u++) st_bounce<STREAM>(bounce + base + u * kThreads, x[u]);
+        }
         grid_complete(cflag, seq, pack_arrive, blockIdx.x, P, 0);
     } else {
         const unsigned bid = blockIdx.x - P, S = gridDim.x - P;
         gate_wait_as(bid, wait_flag, seq, spin_limit, relay, nullptr, false, nullptr, true);
         for (unsigned t = bid; t < tiles; t += S) {
+            if (t == tiles - 1 && (nbytes & (kTileBytes - 1))) {
+                ragged_tile<DT, U, STREAM, false, true>(a, b, bounce, out, (size_t)t * (kThreads * U), nbytes, false);
+                break;
+            }
             const size_t base = (size_t)t * (kThreads * U) + tid;
             u32x4 x[U], y[U];
 #pragma unroll
@@ -638,21 +707,23 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
     // can count the blocks), completion counted on the bounce stores alone
     Geom g = geom_for(p.nbytes, false, true);
     if (g.unroll != 2) g.unroll = 1;
-    // whole tiles, one pass, nothing but the step itself: the stripped kernel
-    if (g.unroll == 2 && g.block == kThreads && !(s.nbytes & 15) && (s.nbytes >> 4) == (size_t)g.grid * kThreads * 2 &&
+    // one pass, nothing but the step itself: the stripped kernel
+    const size_t lean_blocks = (s.nbytes + (size_t)kThreads * 2 * 16 - 1) / ((size_t)kThreads * 2 * 16);
+    if (g.unroll == 2 && g.block == kThreads && lean_blocks <= (size_t)(g_grid_cap_given ? g_grid_cap : kMostBlocks) &&
         s.cflag && !s.pre_word && !s.fp && !s.tagp && !s.done) {
-        const WholeArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid};
+        g.grid = (int)lean_blocks;
+        const LeanArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid, s.nbytes};
         if (g_stream) {
             switch (q.dtype) {
-                case 0: return launch_each(k_fused_whole<0, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
-                case 1: return launch_each(k_fused_whole<1, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
-                default: return launch_each(k_fused_whole<2, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+                case 0: return launch_each(k_fused_lean<0, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+                case 1: return launch_each(k_fused_lean<1, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+                default: return launch_each(k_fused_lean<2, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
             }
         }
         switch (q.dtype) {
-            case 0: return launch_each(k_fused_whole<0, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
-            case 1: return launch_each(k_fused_whole<1, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
-            default: return launch_each(k_fused_whole<2, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+            case 0: return launch_each(k_fused_lean<0, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+            case 1: return launch_each(k_fused_lean<1, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+            default: return launch_each(k_fused_lean<2, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
         }
     }
     if (g_stream) {
@@ -680,32 +751,38 @@ static hipError_t launch_merged_u(const StepArgs& s, int grid, int block, int un
 }
 
 template <int DT, bool STREAM>
-static hipError_t launch_merged_whole(const WholeArgs& w, int grid, int unroll, hipStream_t st, const Timing* t)
+static hipError_t launch_merged_lean(const LeanArgs& w, int grid, int unroll, hipStream_t st, const Timing* t)
 {
-    if (unroll == 2) return launch_each(k_merged_whole<DT, 2, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
-    return launch_each(k_merged_whole<DT, 1, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq);
+    if (unroll == 2) return launch_each(k_merged_lean<DT, 2, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+    return launch_each(k_merged_lean<DT, 1, STREAM>, grid, kThreads, st, t, w.pack_blocks, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
 }
 
 static hipError_t launch_merged_one(int dtype, StepArgs& s, hipStream_t st, const Timing* t)
 {
-    const Geom g = geom_for(s.nbytes, false, true);
+    Geom g = geom_for(s.nbytes, false, true);
+    // each part a multiple of eight blocks long: pack block b and sum block P + b then share an XCD and its L2
+    if (!g_grid_cap_given && g.grid > 8) g.grid = (g.grid + 7) & ~7;
     s.pack_blocks = (unsigned)g.grid;
-    const int grid = 2 * g.grid, u = g.unroll == 8 ? 4 : g.unroll;
-    // whole tiles, one pass, nothing but the step itself: the stripped kernel
-    if ((u == 1 || u == 2) && g.block == kThreads && !(s.nbytes & 15) && (s.nbytes >> 4) == (size_t)g.grid * kThreads * u &&
+    int grid = 2 * g.grid;
+    const int u = g.unroll == 8 ? 4 : g.unroll;
+    // one pass, nothing but the step itself: the stripped kernel (a last tile that is not whole goes to one block's slow path)
+    const size_t lean_blocks = (s.nbytes + (size_t)kThreads * u * 16 - 1) / ((size_t)kThreads * u * 16);
+    if ((u == 1 || u == 2) && g.block == kThreads && lean_blocks <= (size_t)(g_grid_cap_given ? g_grid_cap : kMostBlocks) &&
         s.cflag && s.sigmode == 0 && !s.pre_word && !s.fp && !s.tagp && !s.done) {
-        const WholeArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid};
+        const unsigned part = (unsigned)((lean_blocks + 7) & ~(size_t)7);       // a multiple of eight (so is the cap)
+        grid = 2 * (int)part;
+        const LeanArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, part, s.nbytes};
         if (g_stream) {
             switch (dtype) {
-                case 0: return launch_merged_whole<0, true>(w, grid, u, st, t);
-                case 1: return launch_merged_whole<1, true>(w, grid, u, st, t);
-                default: return launch_merged_whole<2, true>(w, grid, u, st, t);
+                case 0: return launch_merged_lean<0, true>(w, grid, u, st, t);
+                case 1: return launch_merged_lean<1, true>(w, grid, u, st, t);
+                default: return launch_merged_lean<2, true>(w, grid, u, st, t);
             }
         }
         switch (dtype) {
-            case 0: return launch_merged_whole<0, false>(w, grid, u, st, t);
-            case 1: return launch_merged_whole<1, false>(w, grid, u, st, t);
-            default: return launch_merged_whole<2, false>(w, grid, u, st, t);
+            case 0: return launch_merged_lean<0, false>(w, grid, u, st, t);
+            case 1: return launch_merged_lean<1, false>(w, grid, u, st, t);
+            default: return launch_merged_lean<2, false>(w, grid, u, st, t);
         }
     }
     if (g_stream) {
@@ -807,25 +884,29 @@ hipError_t launch_pipe(const PackArgs& p, const SumArgs& q, hipStream_t st, cons
     if (T < 1) T = 1;
     if (T > 0x7fffffffu) return hipErrorInvalidValue;
     const size_t wcap = (size_t)(q.wait_flag ? gated_cap_for(block) : g_grid_cap);
-    const int S = (int)(T < wcap ? T : wcap);
+    int S = (int)(T < wcap ? T : wcap);
     sm.tiles = (unsigned)T;
     pk.pack_blocks = (unsigned)P;
-    // one staged call of whole tiles, out of place, nothing but the step itself: the stripped kernel
+    // one staged call that one pass covers, out of place, nothing but the step itself: the stripped kernel
     if (p.src == q.a && p.nbytes == q.nbytes && !same && q.wait_flag && q.b_uncached && up == 2 && us == 2 && block == kThreads &&
-        !(p.nbytes & 15) && pvec == (size_t)P * kThreads * 2 && !p.pre.word && !q.pre.word && !q.fp && !q.done && !p.fp) {
-        const WholeGateArgs w{WholeArgs{pk.a, sm.b, pk.bounce, sm.out, pk.cflag, pk.pack_arrive, pk.seq, (unsigned)P},
+        (p.nbytes + 8191) / 8192 <= (size_t)pcap && !p.pre.word && !q.pre.word && !q.fp && !q.done && !p.fp) {
+        T = (p.nbytes + 8191) / 8192;                        // tiles of 8 KiB, the last one possibly ragged
+        P = (int)((T + 7) & ~(size_t)7);                      // the pack part a multiple of eight blocks long (pairs on one XCD)
+        S = (int)(T < wcap ? T : wcap);
+        if (S > 8) S &= ~7;
+        const LeanGateArgs w{LeanArgs{pk.a, sm.b, pk.bounce, sm.out, pk.cflag, pk.pack_arrive, pk.seq, (unsigned)P, p.nbytes},
                               q.wait_flag, q.relay, q.spin_limit_ticks, (unsigned)T};
         if (g_stream) {
             switch (q.dtype) {
-                case 0: return launch_each(k_pipe_whole<0, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
-                case 1: return launch_each(k_pipe_whole<1, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
-                default: return launch_each(k_pipe_whole<2, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+                case 0: return launch_each(k_pipe_lean<0, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
+                case 1: return launch_each(k_pipe_lean<1, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
+                default: return launch_each(k_pipe_lean<2, true>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
             }
         }
         switch (q.dtype) {
-            case 0: return launch_each(k_pipe_whole<0, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
-            case 1: return launch_each(k_pipe_whole<1, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
-            default: return launch_each(k_pipe_whole<2, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles);
+            case 0: return launch_each(k_pipe_lean<0, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
+            case 1: return launch_each(k_pipe_lean<1, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
+            default: return launch_each(k_pipe_lean<2, false>, P + S, kThreads, st, t, w.w.pack_blocks, w.w.a, w.w.b, w.w.out, w.relay, w.w.seq, w.w.bounce, w.wait_flag, w.w.cflag, w.w.pack_arrive, w.spin_limit, w.tiles, w.w.nbytes);
         }
     }
     if (g_stream) {

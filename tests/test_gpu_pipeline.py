@@ -312,17 +312,19 @@ def test_resident_peer_merged_launch_ragged(orc, streaming, segment):
 
 
 @pytest.mark.parametrize("streaming", [0, 1])
-def test_resident_peer_in_place_whole_tiles(orc, streaming):
-    """In place (the reference's outp == NULL) with the peer early and a payload of whole tiles: the stripped fused
-    body (one lane loads a vector once, stores it to the bounce and stores the sum over it).  Every call's output
-    equals the oracle's sum AND its bounce image equals the ORIGINAL tensor; then bursts of back-to-back in-place
-    calls on distinct tensors, checked after each burst."""
+def test_resident_peer_stripped_kernels(orc, streaming):
+    """The stripped kernels of the early-peer step at sizes of whole tiles and with a ragged last tile (whole vectors
+    short of a tile, a few odd bytes): out of place (merged launch) and in place (the reference's outp == NULL: the
+    fused body, one lane loads a vector once, stores it to the bounce and stores the sum over it).  Every call's
+    output equals the oracle's sum AND its bounce image equals the ORIGINAL tensor; then bursts of back-to-back
+    in-place calls on distinct tensors, checked after each burst."""
     import ctypes
     hip = ctypes.CDLL("libamdhip64.so.7")
     hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
     cap = 16 << 20
     with session(rails=2, cap=cap, TBV_NSLOT=4, TBV_STREAMING=streaming) as tbv:
-        for name, sizes in (("bf16", (2 << 20, 6 << 20, 8 << 20, 16 << 20)), ("f16", (16 << 20,)), ("f32", (4 << 20, 16 << 20))):
+        for name, sizes in (("bf16", (2 << 20, 6 << 20, 8 << 20, 16 << 20, (8 << 20) + 48, (11 << 20) + 2, (16 << 20) - 6)),
+                            ("f16", (16 << 20, (9 << 20) + 8194)), ("f32", (4 << 20, 16 << 20, (10 << 20) + 4))):
             dt = DT[name]
             esz = 4 if name == "f32" else 2
             peer = dev(synth.uniform(170, cap // esz), dt)
@@ -332,9 +334,16 @@ def test_resident_peer_in_place_whole_tiles(orc, streaming):
                 a = dev(synth.uniform(171 + k, numel), dt)
                 want = oracle_sum(orc, a, peer[:numel])
                 img = torch.empty_like(a)
-                for it in range(6):
+                out = torch.empty_like(a)
+                say("out of place", name, nbytes, "streaming", streaming)
+                assert tbv.all_reduce(a, out)
+                torch.cuda.synchronize()
+                assert first_diff(out, want) is None, (name, nbytes, "out of place")
+                assert hip.hipMemcpy(img.data_ptr(), tbv.lib().tbv_emu_send_slot(tbv.seq() % 4), nbytes, 3) == 0
+                assert np.array_equal(bits_np(img), bits_np(a)), (name, nbytes, "bounce image, out of place")
+                for it in range(4):
                     c = a.clone()
-                    say("in place, whole tiles", name, nbytes, "streaming", streaming, it)
+                    say("in place", name, nbytes, "streaming", streaming, it)
                     assert tbv.all_reduce(c)
                     torch.cuda.synchronize()
                     assert first_diff(c, want) is None, (name, nbytes, it)
@@ -375,7 +384,10 @@ def test_staged_call_in_one_launch(orc, env):
         for name in ("bf16", "f16", "f32"):
             dt = DT[name]
             esz = 4 if name == "f32" else 2
-            sizes = [(1 << 20) // esz + 8, (3 << 20) // esz + 7, (2 << 20) // esz + 3, (5 << 20) // esz - 1] + ([cap // esz] if name == "bf16" else [])
+            # (from 8 MiB the staged launch has a stripped form whose last tile may be ragged: whole vectors short of a
+            # tile, a few odd bytes, and both)
+            sizes = [(1 << 20) // esz + 8, (3 << 20) // esz + 7, (2 << 20) // esz + 3, (5 << 20) // esz - 1,
+                     (9 << 20) // esz + 24, (12 << 20) // esz + 1, (8 << 20) // esz + 4099] + ([cap // esz] if name == "bf16" else [])
             for k, numel in enumerate(sizes):
                 a = dev(synth.uniform(171 + k, numel), dt); p = dev(synth.uniform(271 + k, numel), dt)
                 want = oracle_sum(orc, a, p)
