@@ -274,15 +274,18 @@ __global__ __launch_bounds__(kThreads) void k_merged_lean(unsigned P, const u32x
 // The fused body and the staged launch for the same common case (one pass of tiles of two vectors per lane, no
 // diagnostics, no done word, no earlier kernel's signal).
 template <int DT, bool STREAM>
-__global__ __launch_bounds__(kThreads) void k_fused_lean(const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
+__global__ __launch_bounds__(kThreads) void k_fused_lean(unsigned nblk_ragged, const u32x4* a, const u32x4* b, u32x4* bounce, u32x4* out,
                                                           unsigned long long* cflag, unsigned int* pack_arrive, unsigned long long seq,
                                                           size_t nbytes)
 {
+    // The number of blocks, and in its top bit whether the last tile is ragged, come as the first argument, preloaded
+    // with the pointers: nothing a block has to load (the grid's dimensions, the byte count) stands between its start
+    // and its first data load unless it is that last block.
     constexpr int U = 2;
-    constexpr size_t kTileBytes = (size_t)kThreads * U * 16;
-    if (blockIdx.x == gridDim.x - 1 && (nbytes & (kTileBytes - 1))) {
+    const unsigned nblk = nblk_ragged & 0x7fffffffu;
+    if (nblk_ragged == ((blockIdx.x + 1) | 0x80000000u)) {
         ragged_tile<DT, U, STREAM, true, true>(a, b, bounce, out, (size_t)blockIdx.x * (kThreads * U), nbytes, (const void*)out == (const void*)a);
-        grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0);
+        grid_complete(cflag, seq, pack_arrive, blockIdx.x, nblk, 0);
         return;
     }
     const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
@@ -295,7 +298,7 @@ __global__ __launch_bounds__(kThreads) void k_fused_lean(const u32x4* a, const u
     const bool in_place = (const void*)out == (const void*)a;
 #pragma unroll
     for (int u = 0; u < U; u++) st_out_at<STREAM>(out + base + u * kThreads, add_vec<DT>(x[u], y[u]), in_place);
-    grid_complete(cflag, seq, pack_arrive, blockIdx.x, gridDim.x, 0, U);
+    grid_complete(cflag, seq, pack_arrive, blockIdx.x, nblk, 0, U);
 }
 
 struct LeanGateArgs {
@@ -715,15 +718,15 @@ hipError_t launch_pack_sum(const PackArgs& p, const SumArgs& q, hipStream_t st, 
         const LeanArgs w{s.a, s.b, s.bounce, s.out, s.cflag, s.pack_arrive, s.seq, (unsigned)g.grid, s.nbytes};
         if (g_stream) {
             switch (q.dtype) {
-                case 0: return launch_each(k_fused_lean<0, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
-                case 1: return launch_each(k_fused_lean<1, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
-                default: return launch_each(k_fused_lean<2, true>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+                case 0: return launch_each(k_fused_lean<0, true>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+                case 1: return launch_each(k_fused_lean<1, true>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+                default: return launch_each(k_fused_lean<2, true>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
             }
         }
         switch (q.dtype) {
-            case 0: return launch_each(k_fused_lean<0, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
-            case 1: return launch_each(k_fused_lean<1, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
-            default: return launch_each(k_fused_lean<2, false>, g.grid, kThreads, st, t, w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+            case 0: return launch_each(k_fused_lean<0, false>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+            case 1: return launch_each(k_fused_lean<1, false>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
+            default: return launch_each(k_fused_lean<2, false>, g.grid, kThreads, st, t, w.pack_blocks | ((w.nbytes & 8191) ? 0x80000000u : 0u), w.a, w.b, w.bounce, w.out, w.cflag, w.pack_arrive, w.seq, w.nbytes);
         }
     }
     if (g_stream) {
