@@ -245,12 +245,24 @@ template <unsigned LPG, bool DPP>
 __device__ __forceinline__ void group_minmax(float& mn, float& mx)
 {
     if (DPP) {
-#define TBV_ROR(x, n) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + (n), 0xf, 0xf, false))
-        mn = __builtin_fminf(mn, TBV_ROR(mn, 8)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 8));
-        mn = __builtin_fminf(mn, TBV_ROR(mn, 4)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 4));
-        mn = __builtin_fminf(mn, TBV_ROR(mn, 2)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 2));
-        mn = __builtin_fminf(mn, TBV_ROR(mn, 1)); mx = __builtin_fmaxf(mx, TBV_ROR(mx, 1));
-#undef TBV_ROR
+        // Written out, because the compiler turns each rotation into a move, a canonicalising max and the min (five
+        // instructions a step with their wait states, against one here).  A lane-crossing read needs two wait states
+        // after the write of the register it reads: the other chain's instruction and one s_nop provide them, and
+        // the leading s_nop covers whatever wrote mn, mx or the exec mask just before.  Neither input can be a
+        // signalling NaN (both come out of min/max instructions), so the missing canonicalisation changes nothing.
+        asm("s_nop 4\n\t"
+            "v_min_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+            "v_max_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0\n\t"
+            "v_min_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_max_f32_dpp %1, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0\n\t"
+            "v_min_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_max_f32_dpp %1, %1, %1 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0\n\t"
+            "v_min_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_max_f32_dpp %1, %1, %1 row_ror:1 row_mask:0xf bank_mask:0xf"
+            : "+v"(mn), "+v"(mx));
         if (LPG == 32) {
             mn = __builtin_fminf(mn, __shfl_xor(mn, 16, 64));
             mx = __builtin_fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -328,8 +340,12 @@ __device__ __forceinline__ void coded_work(const StepArgs& g, size_t sb, const C
     }
 }
 
-// (Tried and dropped, 16 MiB bf16 cold, 12.65 us as it stands: two superblocks' loads issued together 13.05; the next
-// superblock's loads issued ahead of the work on the current one, with and without a branch around the loads, 13.7-14.1.
+// (Tried and dropped, 16 MiB bf16 cold, 12.55 us as it stood, 12.45 with the rotations written out: two superblocks'
+// loads issued together 13.05; the next superblock's loads issued ahead of the work on the current one, with and without
+// a branch around the loads, 13.7-14.1 (the compiler's waits at the head of such a loop still cover the stores issued
+// before, whichever way the registers take turns); a branch-free copy of the work for superblocks in which every lane
+// has a vector 13.9; one superblock per block in a stripped kernel with preloaded arguments 12.95 (10.95 against 11.7
+// when the tensors are resident in the cache); the output stored without write-through 12.6.
 // Taking the parts out one at a time says where the time goes: header stores 0.2 us, code stores 1.4, the peer's codes
 // 1.2, decode + sum + output store 2.8, and 7.3 us remain for reading the local tensor and making the codes.)
 template <int DT, bool DPP>
