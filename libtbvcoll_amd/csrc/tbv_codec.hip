@@ -345,7 +345,8 @@ __device__ __forceinline__ void coded_work(const StepArgs& g, size_t sb, const C
 // a branch around the loads, 13.7-14.1 (the compiler's waits at the head of such a loop still cover the stores issued
 // before, whichever way the registers take turns); a branch-free copy of the work for superblocks in which every lane
 // has a vector 13.9; one superblock per block in a stripped kernel with preloaded arguments 12.95 (10.95 against 11.7
-// when the tensors are resident in the cache); the output stored without write-through 12.6.
+// when the tensors are resident in the cache); the output stored without write-through 12.6; blocks that share a CU given
+// different wave priorities or a staggered start 12.65-13.0.
 // Taking the parts out one at a time says where the time goes: header stores 0.2 us, code stores 1.4, the peer's codes
 // 1.2, decode + sum + output store 2.8, and 7.3 us remain for reading the local tensor and making the codes.)
 template <int DT, bool DPP>
